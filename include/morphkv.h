@@ -1,0 +1,255 @@
+/*
+ * morphkv -- C ABI of the MI355X (gfx950) paged-KV hot path.
+ *
+ * One shared library, plain pointers and sizes, no torch types.  Every entry
+ * point returns 0 on success or a negative MKV_E* code (mkv_last_error() gives
+ * the text), never throws, launches on the hipStream_t passed last (as void*),
+ * and does not synchronise unless its name ends in _sync.  All pointers are
+ * device pointers unless the comment says "host".
+ *
+ * Citations name the reference interface each entry point replaces
+ * (MS/ = MorphServe/, CS/ = csrc/src/ in the reference checkout).
+ *
+ * Cache layout everywhere: k_cache, v_cache : [num_blocks, L, Hkv, B, D] fp16,
+ * contiguous, K and V separate (MS/worker/model.py:180-190).  block_table :
+ * [max_seqs, max_blocks_per_seq] int32.
+ */
+#ifndef MORPHKV_H
+#define MORPHKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MKV_OK            0
+#define MKV_EINVAL       -1   /* bad argument / unsupported shape          */
+#define MKV_EHIP         -2   /* a HIP runtime call failed                 */
+#define MKV_ENOSPC       -3   /* not enough free blocks / does not fit     */
+#define MKV_ELOGIC       -4   /* allocator precondition violated           */
+
+#define MKV_MAX_SEGMENTS 128
+
+/*
+ * Where blocks live.  Ids < num_blocks_org address the base pool; an id beyond
+ * it belongs to extension segment (id - org) / seg_blocks at local index
+ * (id - org) % seg_blocks (MS/worker/kernels/kvcache_mgmt.py:169-183,
+ * MS/worker/kernels/paged_attn.py:354-360).  The reference passes segment 0
+ * only and reaches segment j at "- j * org_layer_param_size" elements; the
+ * caller expands that rule into k_seg[j] / v_seg[j] (mkv_pool_set_strided does
+ * it), so any placement of segments is expressible.
+ */
+typedef struct mkv_pool {
+    void*   k_base;
+    void*   v_base;
+    int64_t num_blocks_org;
+    int64_t seg_blocks;        /* S; 0 when there are no segments */
+    int32_t num_segments;
+    int32_t num_layers;        /* L   */
+    int32_t num_kv_heads;      /* Hkv */
+    int32_t block_size;        /* B   */
+    int32_t head_dim;          /* D   */
+    int32_t _pad;
+    void*   k_seg[MKV_MAX_SEGMENTS];
+    void*   v_seg[MKV_MAX_SEGMENTS];
+} mkv_pool;
+
+/* ---- library ---------------------------------------------------------- */
+const char* mkv_last_error(void);           /* host string, thread-local    */
+int  mkv_version(void);
+int  mkv_sizeof_pool(void);                 /* sizeof(mkv_pool), for binding checks */
+/* Fill k_seg/v_seg from the reference's calling convention: segment j at
+ * k_new0 - j * org_layer_param_size * elem_bytes (same for V).
+ * CS/block_swapping.cpp:156-160, MS/worker/kernels/kvcache_mgmt.py:177-183. */
+int  mkv_pool_set_strided(mkv_pool* pool, void* k_new0, void* v_new0,
+                          int64_t org_layer_param_size, int32_t elem_bytes,
+                          int32_t num_segments);
+
+/* ---- KV append -------------------------------------------------------- */
+/* _fwd_kvcache_mgmt_decoding_kernel{,_new_kv_combined},
+ * MS/worker/kernels/kvcache_mgmt.py:52-81, :189-251.
+ * k, v : [n, Hkv, D] fp16; row i is written at position seq_lens[i]-1 of
+ * sequence seq_ids[i]. */
+int mkv_append_decode(const void* k, const void* v, const mkv_pool* pool,
+                      const int32_t* block_table, int64_t max_blocks_per_seq,
+                      const int32_t* seq_ids, const int32_t* seq_lens,
+                      int32_t n, int32_t layer, void* stream);
+
+/* _fwd_kvcache_mgmt_prefill_kernel{,_new_kv_combined},
+ * MS/worker/kernels/kvcache_mgmt.py:12-50, :84-187.
+ * k, v : [num_prefill_tokens, Hkv, D] fp16. */
+int mkv_append_prefill(const void* k, const void* v, const mkv_pool* pool,
+                       const int32_t* block_table, int64_t max_blocks_per_seq,
+                       const int32_t* seq_ids, const int32_t* start_locs,
+                       const int32_t* seq_lens, int32_t num_seqs,
+                       int32_t max_len, int32_t layer, void* stream);
+
+/* ---- paged decode attention -------------------------------------------- */
+/* Scratch the caller must provide for n sequences, Hq heads and up to
+ * max_splits splits: returns bytes for mid_o (fp32 [n,Hq,max_splits,D]) and
+ * mid_lse (fp32 [n,Hq,max_splits]).  Replaces the per-call torch.empty of
+ * MS/worker/kernels/paged_attn.py:780-793. */
+int mkv_paged_attn_scratch_bytes(int32_t n, int32_t num_q_heads, int32_t head_dim,
+                                 int32_t max_splits, int64_t* mid_o_bytes,
+                                 int64_t* mid_lse_bytes);
+
+/* paged_attention = phase 1 + phase 2, MS/worker/kernels/paged_attn.py:59-240,
+ * :243-437, :658-696, :700-1015.  q : [n, Hq, D] fp16, o : [n, Hq, D] fp16.
+ * A sequence is cut into splits of tokens_per_split tokens (a multiple of the
+ * block size); max_splits >= ceil(max_len / tokens_per_split) sizes the scratch
+ * rows.  softmax_scale is 1/sqrt(D); the kernel works in base 2. fp32
+ * accumulation throughout. */
+int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
+                          const int32_t* block_table, int64_t max_blocks_per_seq,
+                          const int32_t* seq_ids, const int32_t* seq_lens,
+                          int32_t n, int32_t num_q_heads, float softmax_scale,
+                          int32_t layer, int32_t tokens_per_split, int32_t max_splits,
+                          void* mid_o, void* mid_lse, void* stream);
+
+/* ---- prefill attention -------------------------------------------------- */
+/* prefill_attention, MS/worker/kernels/prefill_attn.py:9-139, and the live
+ * flash_attn_varlen_func call, MS/worker/layers/transformer_layer.py:154-164:
+ * causal attention of each prefill sequence over its own contiguous q, k, v.
+ * q, o : [T, Hq, D] fp16; k, v : [T, Hkv, D] fp16. */
+int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
+                     const int32_t* start_locs, const int32_t* seq_lens,
+                     int32_t num_seqs, int32_t max_len, int32_t num_q_heads,
+                     int32_t num_kv_heads, int32_t head_dim, float softmax_scale,
+                     void* stream);
+
+/* Chunked prefill over the paged cache.  No counterpart in the reference, which
+ * prefills whole prompts over the batch's own k, v (MS/server/engine.py:259-262,
+ * MS/worker/layers/transformer_layer.py:151-164).  Chunk b holds chunk_lens[b]
+ * query rows at positions prefix_lens[b] .. of sequence seq_ids[b]; K/V of every
+ * position up to the chunk's end are already in the cache (append first); row at
+ * position p attends to cached positions <= p.  prefix_lens may be NULL (= 0). */
+int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
+                           const int32_t* block_table, int64_t max_blocks_per_seq,
+                           const int32_t* seq_ids, const int32_t* start_locs,
+                           const int32_t* chunk_lens, const int32_t* prefix_lens,
+                           int32_t num_seqs, int32_t max_chunk_len, int32_t num_q_heads,
+                           float softmax_scale, int32_t layer, void* stream);
+
+/* ---- block manager ------------------------------------------------------ */
+/* BlockManager.allocate_blocks_for_seqs, MS/worker/block_manager.py:64-112 with
+ * set_block_table_and_num_seq_alloc_blocks, MS/worker/kernels/block_mgmt.py:5-46,
+ * as ONE launch: need_i = ceil(target_lens[i]/B) - n_alloc[seq_ids[i]]; the
+ * sum(need) lowest free ids ascending are marked used, written to new_ids
+ * (int64, capacity new_ids_cap) and appended to the table rows in batch order.
+ * result (3 x int64, device) receives {total_need, status, free_found}; status
+ * 0 ok, MKV_ELOGIC if some need_i < 0 (or a seq id / row length is out of
+ * range), MKV_ENOSPC if fewer than total_need
+ * blocks are free or total_need > new_ids_cap; on a non-zero status no state
+ * is modified. */
+int mkv_bm_allocate(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                    int32_t* block_table, int64_t max_blocks_per_seq,
+                    uint8_t* is_block_free, int64_t num_blocks, const int32_t* seq_ids,
+                    const int32_t* target_lens, int32_t batch, int32_t block_size,
+                    int64_t* new_ids, int64_t new_ids_cap, int64_t* result,
+                    void* stream);
+
+/* torch.nonzero(is_block_free)[:n] + mark used, MS/worker/block_manager.py:75-77.
+ * result (2 x int64, device) receives {found, status}. */
+int mkv_bm_take_first_free(uint8_t* is_block_free, int64_t num_blocks, int64_t n,
+                           int64_t* ids_out, int64_t* result, void* stream);
+
+/* set_block_table_and_num_seq_alloc_blocks, MS/worker/kernels/block_mgmt.py:26-46.
+ * candidate_blocks int64 [sum(block_needed)], block_needed int32 or int64
+ * [batch] (needed_is_i64 selects). */
+int mkv_bt_append(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                  int32_t* block_table, int64_t max_blocks_per_seq,
+                  const int64_t* candidate_blocks,
+                  const int32_t* seq_ids, const void* block_needed,
+                  int32_t needed_is_i64, int32_t batch, void* stream);
+
+/* unset_block_table_and_num_seq_alloc_blocks, MS/worker/kernels/block_mgmt.py:49-80.
+ * freed_total (1 x int64, device, may be NULL) receives sum of released counts. */
+int mkv_bt_release(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                   const int32_t* block_table, int64_t max_blocks_per_seq,
+                   const int32_t* seq_ids, int32_t batch, uint8_t* is_block_free,
+                   int64_t num_blocks, int64_t* freed_total, void* stream);
+
+/* gather_allocated_blocks_and_unset, MS/worker/kernels/block_mgmt.py:83-125.
+ * gathered int32 [capacity]; result (2 x int64, device) receives {total, status}
+ * (MKV_ENOSPC and nothing modified when total > capacity). */
+int mkv_bt_gather_release(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                          const int32_t* block_table, int64_t max_blocks_per_seq,
+                          const int32_t* seq_ids, int32_t batch, uint8_t* is_block_free,
+                          int64_t num_blocks, int32_t* gathered, int64_t capacity,
+                          int64_t* result, void* stream);
+
+/* ---- elastic pool -------------------------------------------------------- */
+/* MemoryManager::acquire_new_kvcache arithmetic, CS/memory_manager.cpp:84-101,
+ * :145 (host, no GPU work): from a weight layer region [layer_base, +org_bytes)
+ * whose first quant_bytes stay in use, the 256-byte aligned K start, the number
+ * of blocks S that fit and the V start.  MKV_ENOSPC when S == 0. */
+int mkv_pool_carve_segment(uint64_t layer_base, uint64_t org_bytes, uint64_t quant_bytes,
+                           int32_t num_layers, int32_t num_kv_heads, int32_t block_size,
+                           int32_t head_dim, uint64_t* k_start, int64_t* seg_blocks,
+                           uint64_t* v_start);
+
+/* k_cache.zero_() / v_cache.zero_() of new pool memory,
+ * CS/memory_manager.cpp:162-163, MS/worker/model.py:189-190. */
+int mkv_fill_zero(void* ptr, uint64_t bytes, void* stream);
+
+/* if_kv_cache_unused, MS/server/memory_utils.py:529-544: result (1 x int64,
+ * device) receives the number of live (not free) blocks in [lo, hi). */
+int mkv_bm_count_live(const uint8_t* is_block_free, int64_t lo, int64_t hi,
+                      int64_t* result, void* stream);
+
+/* Shrink with live-block migration.  No counterpart in the reference, which
+ * refuses to shrink a live tail segment (MS/server/memory_utils.py:623-624).
+ * Plan: src = ascending live ids >= new_num_blocks, dst = the lowest free ids
+ * < new_num_blocks ascending (the allocator's policy,
+ * MS/worker/block_manager.py:75).  Writes src/dst (int64, capacity cap),
+ * remap (int32 [num_blocks], identity except remap[src_k] = dst_k), marks dst
+ * used; result (3 x int64, device) = {moves, status, free_below}.  On
+ * MKV_ENOSPC nothing is modified. */
+int mkv_pool_plan_shrink(uint8_t* is_block_free, int64_t num_blocks,
+                         int64_t new_num_blocks, int64_t* src, int64_t* dst,
+                         int64_t cap, int32_t* remap, int64_t* result, void* stream);
+
+/* Copy K and V of block src[k] to block dst[k], all layers, for k < num_moves
+ * (num_moves read on the host by the caller from mkv_pool_plan_shrink's
+ * result). */
+int mkv_pool_migrate(const mkv_pool* pool, const int64_t* src, const int64_t* dst,
+                     int64_t num_moves, void* stream);
+
+/* Rewrite live table entries bt[s, j < n_alloc[s]] through remap. */
+int mkv_bt_remap(int32_t* block_table, int64_t max_blocks_per_seq,
+                 const int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                 const int32_t* remap, int64_t num_blocks, void* stream);
+
+/* ---- eviction ------------------------------------------------------------ */
+/* swap_blocks / swap_blocks_new_kv_combined, CS/block_swapping.cpp:22-85,
+ * :88-202.  src_ids/dst_ids are HOST arrays; k_swap/v_swap are HOST tensors
+ * [num_cpu_blocks, L, Hkv, B, D] fp16.  Runs of consecutive ids (same segment
+ * on the device side) become one hipMemcpyAsync pair; return codes are
+ * checked.  Swap-in writes device block dst_ids[i] from host block src_ids[i].
+ * num_copies (host, may be NULL) receives the number of memcpy pairs issued. */
+int mkv_swap_blocks(const int64_t* src_ids, const int64_t* dst_ids, int64_t count,
+                    int32_t is_swap_in, const mkv_pool* pool, void* k_swap,
+                    void* v_swap, int64_t* num_copies, void* stream);
+
+/* ---- measurement ---------------------------------------------------------- */
+/* Kernel ids for mkv_prof_*. */
+#define MKV_K_APPEND_DECODE   0
+#define MKV_K_APPEND_PREFILL  1
+#define MKV_K_ATTN_PHASE1     2
+#define MKV_K_ATTN_PHASE2     3
+#define MKV_K_MIGRATE         4
+#define MKV_K_PREFILL_ATTN    5
+#define MKV_K_FILL_ZERO       6
+#define MKV_K_COUNT           7
+/* When enabled, every launch of the kernels above is bracketed by a
+ * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
+ * returns the launch count and summed duration since the last reset. */
+int mkv_prof_enable(int32_t on);
+int mkv_prof_reset(void);
+int mkv_prof_collect(int32_t kernel_id, int64_t* launches, double* total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MORPHKV_H */

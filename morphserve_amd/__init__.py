@@ -1,0 +1,24 @@
+"""MI355X-native paged-KV hot path behind the SwiftLLM/MorphServe operator surface.
+
+Drop-in names (reference file each mirrors):
+
+* ``worker.kernels.kvcache_mgmt.store_kvcache``      MorphServe/worker/kernels/kvcache_mgmt.py
+* ``worker.kernels.paged_attn.paged_attention``      MorphServe/worker/kernels/paged_attn.py
+* ``worker.kernels.prefill_attn.prefill_attention``  MorphServe/worker/kernels/prefill_attn.py
+* ``worker.kernels.block_mgmt.*``                    MorphServe/worker/kernels/block_mgmt.py
+* ``worker.block_manager.BlockManager``              MorphServe/worker/block_manager.py
+* ``worker.infer_state.LlamaInferState``             MorphServe/worker/infer_state.py
+* ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
+* ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
+
+All compute goes through ``libmorphkv.so`` (hand-written HIP for gfx950) via
+ctypes; nothing here falls back to eager PyTorch.
+"""
+from . import _capi  # noqa: F401
+from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
+from .worker.block_manager import BlockManager  # noqa: F401
+from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
+from .worker.kernels.paged_attn import paged_attention  # noqa: F401
+from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401
+from .elastic_pool import ElasticKVPool  # noqa: F401
+from . import swiftllm_c  # noqa: F401

@@ -1,0 +1,489 @@
+// Block manager on the device: first-free allocation (ascending lowest ids, the
+// order torch.nonzero would give), block-table append / release / gather, live
+// counts.  Every operation is ONE single-workgroup launch: the state is small
+// (one byte per block, a few ints per sequence), the work is ordered scans, and
+// a single workgroup keeps them deterministic without atomics or host round
+// trips between the steps.
+#include "common.h"
+
+namespace mkv {
+
+static constexpr int kScanThreads = 1024;
+static constexpr int kScanWaves = kScanThreads / 64;
+static constexpr int kBytesPerThread = 16;
+static constexpr int64_t kTileBytes = (int64_t)kScanThreads * kBytesPerThread;
+
+// Exclusive prefix sum over the workgroup (1024 threads); total returned in *total.
+// All threads must call it.
+__device__ __forceinline__ int64_t block_excl_scan(int64_t v, int64_t* total, int64_t* sm /* [kScanWaves + 1] */) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int64_t inc = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int64_t t = __shfl_up(inc, d);
+        if (lane >= d) inc += t;
+    }
+    __syncthreads();                       // sm reuse across calls
+    if (lane == 63) sm[wave] = inc;
+    __syncthreads();
+    if (wave == 0) {
+        int64_t w = lane < kScanWaves ? sm[lane] : 0;
+        int64_t winc = w;
+#pragma unroll
+        for (int d = 1; d < kScanWaves; d <<= 1) {
+            int64_t t = __shfl_up(winc, d);
+            if (lane >= d) winc += t;
+        }
+        if (lane < kScanWaves) sm[lane] = winc - w;       // exclusive wave offsets
+        if (lane == kScanWaves - 1) sm[kScanWaves] = winc;
+    }
+    __syncthreads();
+    *total = sm[kScanWaves];
+    return sm[wave] + inc - v;
+}
+
+// Counts bytes equal to `want` in map[lo, hi) until at least `limit` are seen
+// (early exit at tile granularity).  All threads must call it.
+__device__ int64_t count_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8_t want,
+                               int64_t limit, int64_t* sm) {
+    int64_t seen = 0;
+    for (int64_t t0 = lo; t0 < hi && seen < limit; t0 += kTileBytes) {
+        const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
+        int64_t c = 0;
+#pragma unroll
+        for (int k = 0; k < kBytesPerThread; ++k) {
+            const int64_t b = b0 + k;
+            if (b < hi) c += ((map[b] != 0) == (want != 0));
+        }
+        int64_t tot;
+        block_excl_scan(c, &tot, sm);
+        seen += tot;
+    }
+    return seen;
+}
+
+// Writes the first `n` positions of map[lo, hi) whose byte equals `want` (in
+// ascending order) to out[0..n) and stores `mark` there.  The caller has
+// verified that at least n exist.  All threads must call it.
+__device__ void take_bytes(uint8_t* map, int64_t lo, int64_t hi, uint8_t want, uint8_t mark,
+                           int64_t n, int64_t* out, int64_t* sm) {
+    int64_t base = 0;
+    for (int64_t t0 = lo; t0 < hi && base < n; t0 += kTileBytes) {
+        const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
+        uint32_t bits = 0;
+        int64_t c = 0;
+#pragma unroll
+        for (int k = 0; k < kBytesPerThread; ++k) {
+            const int64_t b = b0 + k;
+            if (b < hi && ((map[b] != 0) == (want != 0))) {
+                bits |= 1u << k;
+                ++c;
+            }
+        }
+        int64_t tot;
+        int64_t pos = base + block_excl_scan(c, &tot, sm);
+#pragma unroll
+        for (int k = 0; k < kBytesPerThread; ++k) {
+            if ((bits >> k) & 1u) {
+                if (pos < n) {
+                    out[pos] = b0 + k;
+                    map[b0 + k] = mark;
+                }
+                ++pos;
+            }
+        }
+        base += tot;
+    }
+}
+
+// ---- allocate_blocks_for_seqs, fused ---------------------------------------------
+__global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
+    int32_t* __restrict__ n_alloc, int32_t* __restrict__ block_table, int64_t max_blocks_per_seq,
+    uint8_t* __restrict__ is_free, int64_t num_blocks, const int32_t* __restrict__ seq_ids,
+    const int32_t* __restrict__ target_lens, int32_t batch, int32_t block_size,
+    int64_t* __restrict__ new_ids, int64_t new_ids_cap, int64_t* __restrict__ result,
+    int64_t max_seqs) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    __shared__ int s_bad;
+    const int tid = threadIdx.x;
+    if (tid == 0) s_bad = 0;
+    __syncthreads();
+
+    // pass 1: total need, precondition need_i >= 0 and room in the table row
+    int64_t my_need = 0;
+    for (int i = tid; i < batch; i += kScanThreads) {
+        const int64_t target = ((int64_t)target_lens[i] + block_size - 1) / block_size;
+        const int64_t seq = seq_ids[i];
+        if (seq < 0 || seq >= max_seqs) { s_bad = 1; continue; }
+        const int64_t have = n_alloc[seq];
+        const int64_t need = target - have;
+        if (need < 0 || target > max_blocks_per_seq) s_bad = 1;
+        my_need += need;
+    }
+    int64_t total;
+    block_excl_scan(my_need, &total, sm);
+    __syncthreads();
+    if (s_bad) {
+        if (tid == 0) { result[0] = total; result[1] = MKV_ELOGIC; result[2] = 0; }
+        return;
+    }
+    if (total == 0) {
+        if (tid == 0) { result[0] = 0; result[1] = MKV_OK; result[2] = 0; }
+        return;
+    }
+    // pass 2: are there enough free blocks? (no state touched yet)
+    const int64_t found = count_bytes(is_free, 0, num_blocks, 1, total, sm);
+    if (found < total || total > new_ids_cap) {
+        if (tid == 0) { result[0] = total; result[1] = MKV_ENOSPC; result[2] = found; }
+        return;
+    }
+    // pass 3: take the lowest `total` free ids
+    take_bytes(is_free, 0, num_blocks, 1, 0, total, new_ids, sm);
+    __threadfence_block();
+    __syncthreads();
+    // pass 4: hand them to the rows in batch order
+    int64_t base = 0;
+    for (int i0 = 0; i0 < batch; i0 += kScanThreads) {
+        const int i = i0 + tid;
+        int64_t need = 0, have = 0, seq = 0;
+        if (i < batch) {
+            seq = seq_ids[i];
+            have = n_alloc[seq];
+            need = ((int64_t)target_lens[i] + block_size - 1) / block_size - have;
+        }
+        int64_t tot;
+        const int64_t start = base + block_excl_scan(need, &tot, sm);
+        if (i < batch && need > 0) {
+            int32_t* dst = block_table + seq * max_blocks_per_seq + have;
+            for (int64_t x = 0; x < need; ++x) dst[x] = (int32_t)new_ids[start + x];
+            n_alloc[seq] = (int32_t)(have + need);
+        }
+        base += tot;
+    }
+    if (tid == 0) { result[0] = total; result[1] = MKV_OK; result[2] = found; }
+}
+
+__global__ __launch_bounds__(kScanThreads) void bm_take_first_free_kernel(
+    uint8_t* __restrict__ is_free, int64_t num_blocks, int64_t n, int64_t* __restrict__ ids_out,
+    int64_t* __restrict__ result) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int64_t found = count_bytes(is_free, 0, num_blocks, 1, n, sm);
+    if (found < n) {
+        if (threadIdx.x == 0) { result[0] = found; result[1] = MKV_ENOSPC; }
+        return;
+    }
+    take_bytes(is_free, 0, num_blocks, 1, 0, n, ids_out, sm);
+    if (threadIdx.x == 0) { result[0] = n; result[1] = MKV_OK; }
+}
+
+template <typename NeedT>
+__global__ __launch_bounds__(kScanThreads) void bt_append_kernel(
+    int32_t* __restrict__ n_alloc, int32_t* __restrict__ block_table, int64_t max_blocks_per_seq,
+    const int64_t* __restrict__ cand, const int32_t* __restrict__ seq_ids,
+    const NeedT* __restrict__ needed, int32_t batch, int64_t max_seqs) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int tid = threadIdx.x;
+    int64_t base = 0;
+    for (int i0 = 0; i0 < batch; i0 += kScanThreads) {
+        const int i = i0 + tid;
+        int64_t need = 0, have = 0, seq = 0;
+        bool ok = false;
+        if (i < batch) {
+            seq = seq_ids[i];
+            ok = seq >= 0 && seq < max_seqs;                   // rows naming no sequence are skipped
+            if (ok) have = n_alloc[seq];
+            need = (int64_t)needed[i];
+            if (need < 0) need = 0;
+        }
+        int64_t tot;
+        const int64_t start = base + block_excl_scan(need, &tot, sm);
+        if (ok && need > 0) {
+            const int64_t fit = min(need, max_blocks_per_seq - have);   // never write past the row
+            int32_t* dst = block_table + seq * max_blocks_per_seq + have;
+            for (int64_t x = 0; x < fit; ++x) dst[x] = (int32_t)cand[start + x];
+            n_alloc[seq] = (int32_t)(have + need);
+        }
+        base += tot;
+    }
+}
+
+// One wave per row at a time; lanes stride over the row's live entries.
+__global__ __launch_bounds__(kScanThreads) void bt_release_kernel(
+    int32_t* __restrict__ n_alloc, const int32_t* __restrict__ block_table,
+    int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids, int32_t batch,
+    uint8_t* __restrict__ is_free, int64_t* __restrict__ freed_total, int64_t max_seqs,
+    int64_t num_blocks) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int64_t mine = 0;
+    for (int i = wave; i < batch; i += kScanWaves) {
+        const int64_t seq = seq_ids[i];
+        if (seq < 0 || seq >= max_seqs) continue;
+        const int32_t cnt = n_alloc[seq];
+        const int32_t* row = block_table + seq * max_blocks_per_seq;
+        for (int j = lane; j < cnt; j += 64) {
+            const int64_t id = row[j];
+            if (id >= 0 && id < num_blocks) is_free[id] = 1;
+        }
+        if (lane == 0) mine += cnt;
+    }
+    __syncthreads();                      // every wave has read the counts it needs
+    for (int i = wave; i < batch; i += kScanWaves) {
+        const int64_t seq = seq_ids[i];
+        if (lane == 0 && seq >= 0 && seq < max_seqs) n_alloc[seq] = 0;
+    }
+    int64_t tot;
+    block_excl_scan(mine, &tot, sm);
+    if (threadIdx.x == 0 && freed_total) *freed_total = tot;
+}
+
+__global__ __launch_bounds__(kScanThreads) void bt_gather_release_kernel(
+    int32_t* __restrict__ n_alloc, const int32_t* __restrict__ block_table,
+    int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids, int32_t batch,
+    uint8_t* __restrict__ is_free, int32_t* __restrict__ gathered, int64_t capacity,
+    int64_t* __restrict__ result, int64_t max_seqs, int64_t num_blocks) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int tid = threadIdx.x;
+    auto count_of = [&](int i) -> int64_t {
+        const int64_t seq = seq_ids[i];
+        return (seq >= 0 && seq < max_seqs) ? (int64_t)n_alloc[seq] : 0;
+    };
+    // total first: nothing is modified when it does not fit
+    int64_t mine = 0;
+    for (int i = tid; i < batch; i += kScanThreads) mine += count_of(i);
+    int64_t total;
+    block_excl_scan(mine, &total, sm);
+    __syncthreads();
+    if (total > capacity) {
+        if (tid == 0) { result[0] = total; result[1] = MKV_ENOSPC; }
+        return;
+    }
+    // Rows are copied one wave at a time; the start offset of row i is the sum of
+    // the counts of the rows before it (seq-major, logical block order).
+    int64_t base = 0;
+    for (int i0 = 0; i0 < batch; i0 += kScanThreads) {
+        const int i = i0 + tid;
+        const int64_t cnt = (i < batch) ? count_of(i) : 0;
+        int64_t tot;
+        const int64_t start = base + block_excl_scan(cnt, &tot, sm);
+        // the thread that owns row i copies it (rows are short: ceil(len/B) entries)
+        if (i < batch && cnt > 0) {
+            const int64_t seq = seq_ids[i];
+            const int32_t* row = block_table + seq * max_blocks_per_seq;
+            for (int64_t x = 0; x < cnt; ++x) {
+                const int32_t id = row[x];
+                gathered[start + x] = id;
+                if (id >= 0 && id < num_blocks) is_free[id] = 1;
+            }
+        }
+        base += tot;
+    }
+    __syncthreads();
+    for (int i = tid; i < batch; i += kScanThreads) {
+        const int64_t seq = seq_ids[i];
+        if (seq >= 0 && seq < max_seqs) n_alloc[seq] = 0;
+    }
+    if (tid == 0) { result[0] = total; result[1] = MKV_OK; }
+}
+
+__global__ __launch_bounds__(kScanThreads) void bm_count_live_kernel(
+    const uint8_t* __restrict__ is_free, int64_t lo, int64_t hi, int64_t* __restrict__ result) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int64_t live = count_bytes(is_free, lo, hi, 0, INT64_MAX, sm);
+    if (threadIdx.x == 0) *result = live;
+}
+
+// ---- shrink planning ---------------------------------------------------------------
+__global__ __launch_bounds__(kScanThreads) void pool_plan_shrink_kernel(
+    uint8_t* __restrict__ is_free, int64_t num_blocks, int64_t new_n, int64_t* __restrict__ src,
+    int64_t* __restrict__ dst, int64_t cap, int32_t* __restrict__ remap,
+    int64_t* __restrict__ result) {
+    __shared__ int64_t sm[kScanWaves + 1];
+    const int tid = threadIdx.x;
+    const int64_t moves = count_bytes(is_free, new_n, num_blocks, 0, INT64_MAX, sm);
+    const int64_t free_below = count_bytes(is_free, 0, new_n, 1, moves, sm);
+    if (free_below < moves || moves > cap) {
+        if (tid == 0) { result[0] = moves; result[1] = MKV_ENOSPC; result[2] = free_below; }
+        return;
+    }
+    for (int64_t b = tid; b < num_blocks; b += kScanThreads) remap[b] = (int32_t)b;
+    // live ids >= new_n ascending become free; lowest free ids < new_n become used
+    take_bytes(is_free, new_n, num_blocks, 0, 1, moves, src, sm);
+    take_bytes(is_free, 0, new_n, 1, 0, moves, dst, sm);
+    __threadfence_block();
+    __syncthreads();
+    for (int64_t k = tid; k < moves; k += kScanThreads) remap[src[k]] = (int32_t)dst[k];
+    if (tid == 0) { result[0] = moves; result[1] = MKV_OK; result[2] = free_below; }
+}
+
+__global__ __launch_bounds__(256) void bt_remap_kernel(int32_t* __restrict__ block_table,
+                                                       int64_t max_blocks_per_seq,
+                                                       const int32_t* __restrict__ n_alloc,
+                                                       int64_t max_seqs,
+                                                       const int32_t* __restrict__ remap,
+                                                       int64_t num_blocks) {
+    for (int64_t row = blockIdx.x; row < max_seqs; row += gridDim.x) {
+        const int32_t cnt = n_alloc[row];
+        int32_t* r = block_table + row * max_blocks_per_seq;
+        for (int j = threadIdx.x; j < cnt; j += blockDim.x) {
+            const int32_t id = r[j];
+            if (id >= 0 && id < num_blocks) {
+                const int32_t to = remap[id];
+                if (to != id) r[j] = to;
+            }
+        }
+    }
+}
+
+}  // namespace mkv
+
+extern "C" {
+
+int mkv_bm_allocate(int32_t* num_seq_allocated_blocks, int64_t max_seqs, int32_t* block_table,
+                    int64_t max_blocks_per_seq, uint8_t* is_block_free, int64_t num_blocks,
+                    const int32_t* seq_ids, const int32_t* target_lens, int32_t batch,
+                    int32_t block_size, int64_t* new_ids, int64_t new_ids_cap, int64_t* result,
+                    void* stream) {
+    MKV_REQUIRE(num_seq_allocated_blocks && block_table && is_block_free && result, "NULL argument");
+    MKV_REQUIRE(batch >= 0 && block_size > 0 && num_blocks >= 0 && max_blocks_per_seq > 0, "bad sizes");
+    MKV_REQUIRE(batch == 0 || (seq_ids && target_lens), "NULL seq_ids/target_lens");
+    MKV_REQUIRE(new_ids || new_ids_cap == 0, "new_ids is NULL");
+    hipLaunchKernelGGL(mkv::bm_allocate_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, num_seq_allocated_blocks, block_table,
+                       max_blocks_per_seq, is_block_free, num_blocks, seq_ids, target_lens, batch,
+                       block_size, new_ids, new_ids_cap, result, max_seqs);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bm_take_first_free(uint8_t* is_block_free, int64_t num_blocks, int64_t n,
+                           int64_t* ids_out, int64_t* result, void* stream) {
+    MKV_REQUIRE(is_block_free && result, "NULL argument");
+    MKV_REQUIRE(n >= 0 && num_blocks >= 0, "bad sizes");
+    MKV_REQUIRE(ids_out || n == 0, "ids_out is NULL");
+    hipLaunchKernelGGL(mkv::bm_take_first_free_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, is_block_free, num_blocks, n, ids_out, result);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bt_append(int32_t* num_seq_allocated_blocks, int64_t max_seqs, int32_t* block_table,
+                  int64_t max_blocks_per_seq, const int64_t* candidate_blocks,
+                  const int32_t* seq_ids, const void* block_needed, int32_t needed_is_i64,
+                  int32_t batch, void* stream) {
+    MKV_REQUIRE(batch >= 0, "batch must be >= 0");
+    if (batch == 0) return MKV_OK;
+    MKV_REQUIRE(num_seq_allocated_blocks && block_table && seq_ids && block_needed, "NULL argument");
+    if (needed_is_i64) {
+        hipLaunchKernelGGL(mkv::bt_append_kernel<int64_t>, dim3(1), dim3(mkv::kScanThreads), 0,
+                           (hipStream_t)stream, num_seq_allocated_blocks, block_table,
+                           max_blocks_per_seq, candidate_blocks, seq_ids,
+                           (const int64_t*)block_needed, batch, max_seqs);
+    } else {
+        hipLaunchKernelGGL(mkv::bt_append_kernel<int32_t>, dim3(1), dim3(mkv::kScanThreads), 0,
+                           (hipStream_t)stream, num_seq_allocated_blocks, block_table,
+                           max_blocks_per_seq, candidate_blocks, seq_ids,
+                           (const int32_t*)block_needed, batch, max_seqs);
+    }
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bt_release(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                   const int32_t* block_table, int64_t max_blocks_per_seq,
+                   const int32_t* seq_ids, int32_t batch, uint8_t* is_block_free,
+                   int64_t num_blocks, int64_t* freed_total, void* stream) {
+    MKV_REQUIRE(batch >= 0, "batch must be >= 0");
+    MKV_REQUIRE(num_seq_allocated_blocks && block_table && is_block_free, "NULL argument");
+    MKV_REQUIRE(batch == 0 || seq_ids, "seq_ids is NULL");
+    hipLaunchKernelGGL(mkv::bt_release_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, num_seq_allocated_blocks, block_table,
+                       max_blocks_per_seq, seq_ids, batch, is_block_free, freed_total, max_seqs,
+                       num_blocks);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bt_gather_release(int32_t* num_seq_allocated_blocks, int64_t max_seqs,
+                          const int32_t* block_table, int64_t max_blocks_per_seq,
+                          const int32_t* seq_ids, int32_t batch, uint8_t* is_block_free,
+                          int64_t num_blocks, int32_t* gathered, int64_t capacity,
+                          int64_t* result, void* stream) {
+    MKV_REQUIRE(batch >= 0 && capacity >= 0, "bad sizes");
+    MKV_REQUIRE(num_seq_allocated_blocks && block_table && is_block_free && result, "NULL argument");
+    MKV_REQUIRE(batch == 0 || seq_ids, "seq_ids is NULL");
+    MKV_REQUIRE(gathered || capacity == 0, "gathered is NULL");
+    hipLaunchKernelGGL(mkv::bt_gather_release_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, num_seq_allocated_blocks, block_table,
+                       max_blocks_per_seq, seq_ids, batch, is_block_free, gathered, capacity,
+                       result, max_seqs, num_blocks);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bm_count_live(const uint8_t* is_block_free, int64_t lo, int64_t hi, int64_t* result,
+                      void* stream) {
+    MKV_REQUIRE(is_block_free && result, "NULL argument");
+    MKV_REQUIRE(0 <= lo && lo <= hi, "need 0 <= lo <= hi");
+    hipLaunchKernelGGL(mkv::bm_count_live_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, is_block_free, lo, hi, result);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_pool_plan_shrink(uint8_t* is_block_free, int64_t num_blocks, int64_t new_num_blocks,
+                         int64_t* src, int64_t* dst, int64_t cap, int32_t* remap,
+                         int64_t* result, void* stream) {
+    MKV_REQUIRE(is_block_free && remap && result, "NULL argument");
+    MKV_REQUIRE(0 <= new_num_blocks && new_num_blocks <= num_blocks,
+                "need 0 <= new_num_blocks (%lld) <= num_blocks (%lld)", (long long)new_num_blocks,
+                (long long)num_blocks);
+    MKV_REQUIRE(num_blocks <= INT32_MAX, "block ids must fit int32");
+    MKV_REQUIRE((src && dst) || cap == 0, "src/dst are NULL");
+    hipLaunchKernelGGL(mkv::pool_plan_shrink_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
+                       (hipStream_t)stream, is_block_free, num_blocks, new_num_blocks, src, dst,
+                       cap, remap, result);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_bt_remap(int32_t* block_table, int64_t max_blocks_per_seq,
+                 const int32_t* num_seq_allocated_blocks, int64_t max_seqs, const int32_t* remap,
+                 int64_t num_blocks, void* stream) {
+    MKV_REQUIRE(block_table && num_seq_allocated_blocks && remap, "NULL argument");
+    MKV_REQUIRE(max_seqs >= 0 && max_blocks_per_seq > 0, "bad sizes");
+    if (max_seqs == 0) return MKV_OK;
+    const unsigned grid = (unsigned)(max_seqs < 65535 ? max_seqs : 65535);
+    hipLaunchKernelGGL(mkv::bt_remap_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
+                       block_table, max_blocks_per_seq, num_seq_allocated_blocks, max_seqs, remap,
+                       num_blocks);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_pool_carve_segment(uint64_t layer_base, uint64_t org_bytes, uint64_t quant_bytes,
+                           int32_t num_layers, int32_t num_kv_heads, int32_t block_size,
+                           int32_t head_dim, uint64_t* k_start, int64_t* seg_blocks,
+                           uint64_t* v_start) {
+    MKV_REQUIRE(k_start && seg_blocks && v_start, "output pointers are NULL");
+    MKV_REQUIRE(num_layers > 0 && num_kv_heads > 0 && block_size > 0 && head_dim > 0, "bad dims");
+    const uint64_t layer_end = layer_base + quant_bytes;
+    const uint64_t start = (layer_end + 255) & ~(uint64_t)255;
+    const uint64_t used = start - layer_base;
+    const uint64_t kv_slot = 2ull * num_layers * num_kv_heads * head_dim * 2ull;
+    const uint64_t kv_block = kv_slot * block_size;
+    const uint64_t avail = org_bytes > used ? org_bytes - used : 0;
+    const uint64_t S = avail / kv_block;
+    if (S == 0) {
+        mkv::set_error("No space available for new KV cache blocks");
+        return MKV_ENOSPC;
+    }
+    *k_start = start;
+    *seg_blocks = (int64_t)S;
+    *v_start = start + S * (kv_block / 2);
+    return MKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,77 @@
+// Shared host/device helpers for the morphkv HIP library (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "morphkv.h"
+
+namespace mkv {
+
+// ---- host-side error plumbing ---------------------------------------------
+void set_error(const char* fmt, ...);
+int  hip_fail(hipError_t e, const char* what);
+
+#define MKV_HIP(call)                                             \
+    do {                                                          \
+        hipError_t _e = (call);                                   \
+        if (_e != hipSuccess) return ::mkv::hip_fail(_e, #call);  \
+    } while (0)
+
+#define MKV_REQUIRE(cond, ...)                                    \
+    do {                                                          \
+        if (!(cond)) {                                            \
+            ::mkv::set_error(__VA_ARGS__);                        \
+            return MKV_EINVAL;                                    \
+        }                                                         \
+    } while (0)
+
+int  check_pool(const mkv_pool* p);
+
+// Brackets one launch with an event pair when profiling is on.
+struct ProfScope {
+    int kernel_id;
+    hipStream_t stream;
+    void* rec;
+    ProfScope(int kernel_id, hipStream_t s);
+    ~ProfScope();
+};
+
+// ---- device-side pool addressing ---------------------------------------------
+// Byte offset of a block inside its pool/segment and the K/V bases it is
+// relative to.  Block ids below num_blocks_org live in the base pool; others in
+// segment (id-org)/S at local index (id-org)%S.
+struct BlockAddr {
+    const char* k;
+    const char* v;
+};
+
+__device__ __forceinline__ BlockAddr block_addr(const mkv_pool& p, int64_t id, int64_t block_bytes) {
+    BlockAddr a;
+    if (id < p.num_blocks_org) {
+        a.k = (const char*)p.k_base + id * block_bytes;
+        a.v = (const char*)p.v_base + id * block_bytes;
+    } else {
+        int64_t rel = id - p.num_blocks_org;
+        int64_t seg = rel / p.seg_blocks;
+        int64_t local = rel - seg * p.seg_blocks;
+        a.k = (const char*)p.k_seg[seg] + local * block_bytes;
+        a.v = (const char*)p.v_seg[seg] + local * block_bytes;
+    }
+    return a;
+}
+
+__host__ __device__ __forceinline__ int64_t pool_block_bytes(const mkv_pool& p) {
+    return (int64_t)p.num_layers * p.num_kv_heads * p.block_size * p.head_dim * 2;
+}
+
+// Ids outside [0, total) would address memory outside the pool; kernels skip them.
+__host__ __device__ __forceinline__ int64_t pool_total_blocks(const mkv_pool& p) {
+    return p.num_blocks_org + (int64_t)p.num_segments * p.seg_blocks;
+}
+
+static inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+}  // namespace mkv

@@ -1,0 +1,180 @@
+// Bulk HBM movers of the elastic pool: live-block migration (batched block copy),
+// zero fill of new pool memory, and host<->device block eviction.
+#include "common.h"
+
+#include <vector>
+
+namespace mkv {
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+static constexpr int kCopyThreads = 256;
+static constexpr int kCopyUnroll = 4;                                   // 16-byte units per thread per chunk
+static constexpr int64_t kChunkBytes = (int64_t)kCopyThreads * kCopyUnroll * 16;   // 16 KiB
+
+// Work item w = (move, K|V, chunk) in that order of significance; a persistent
+// grid strides over the items.  Within a chunk every wave instruction moves
+// 1 KiB of contiguous bytes (16 bytes per lane), loads first, then stores.
+__global__ __launch_bounds__(kCopyThreads) void pool_migrate_kernel(
+    const mkv_pool pool, const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
+    int64_t num_moves, int64_t block_bytes, int32_t chunks_per_block) {
+    const int64_t total_blocks = pool_total_blocks(pool);
+    const int64_t items = num_moves * 2 * chunks_per_block;
+    for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
+        const int64_t mv = w / (2 * chunks_per_block);
+        const int rem = (int)(w - mv * 2 * chunks_per_block);
+        const int is_v = rem / chunks_per_block;
+        const int chunk = rem - is_v * chunks_per_block;
+        const int64_t s = src[mv];
+        const int64_t d = dst[mv];
+        if (s < 0 || s >= total_blocks || d < 0 || d >= total_blocks) continue;
+        BlockAddr sa = block_addr(pool, s, block_bytes);
+        BlockAddr da = block_addr(pool, d, block_bytes);
+        const int64_t off = (int64_t)chunk * kChunkBytes;
+        const uint4* sp = (const uint4*)((is_v ? sa.v : sa.k) + off) + threadIdx.x;
+        uint4* dp = (uint4*)(const_cast<char*>(is_v ? da.v : da.k) + off) + threadIdx.x;
+        const int64_t left = block_bytes - off;                         // bytes left in this block
+        if (left >= kChunkBytes) {
+            v4u r[kCopyUnroll];
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) r[u] = __builtin_nontemporal_load((const v4u*)sp + u * kCopyThreads);
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(r[u], (v4u*)dp + u * kCopyThreads);
+        } else {
+            const int64_t units = left >> 4;                            // block_bytes is a multiple of 16
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) {
+                const int64_t idx = (int64_t)u * kCopyThreads + threadIdx.x;
+                if (idx < units) dp[u * kCopyThreads] = sp[u * kCopyThreads];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, int64_t units,
+                                                        uint8_t* __restrict__ tail, int tail_bytes) {
+    const v4u z = {0u, 0u, 0u, 0u};
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < units; i += stride)
+        __builtin_nontemporal_store(z, (v4u*)p + i);
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail_bytes) tail[threadIdx.x] = 0;
+}
+
+static int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+}  // namespace mkv
+
+extern "C" {
+
+int mkv_pool_migrate(const mkv_pool* pool, const int64_t* src, const int64_t* dst,
+                     int64_t num_moves, void* stream) {
+    int rc = mkv::check_pool(pool);
+    if (rc) return rc;
+    MKV_REQUIRE(num_moves >= 0, "num_moves must be >= 0");
+    if (num_moves == 0) return MKV_OK;
+    MKV_REQUIRE(src && dst, "src/dst are NULL");
+    const int64_t block_bytes = mkv::pool_block_bytes(*pool);
+    const int chunks = mkv::cdiv(block_bytes, mkv::kChunkBytes);
+    const int64_t items = num_moves * 2 * chunks;
+    const int64_t want = (int64_t)mkv::num_cus() * 16;
+    const unsigned grid = (unsigned)(items < want ? items : want);
+    hipStream_t s = (hipStream_t)stream;
+    {
+        mkv::ProfScope prof(MKV_K_MIGRATE, s);
+        hipLaunchKernelGGL(mkv::pool_migrate_kernel, dim3(grid), dim3(mkv::kCopyThreads), 0, s,
+                           *pool, src, dst, num_moves, block_bytes, chunks);
+    }
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_fill_zero(void* ptr, uint64_t bytes, void* stream) {
+    if (bytes == 0) return MKV_OK;
+    MKV_REQUIRE(ptr != nullptr, "ptr is NULL");
+    MKV_REQUIRE(((uintptr_t)ptr & 15) == 0, "ptr must be 16-byte aligned");
+    const int64_t units = (int64_t)(bytes >> 4);
+    const int tail = (int)(bytes & 15);
+    int64_t want = (units + 255) / 256;
+    const int64_t cap = (int64_t)mkv::num_cus() * 16;
+    if (want > cap) want = cap;
+    if (want < 1) want = 1;
+    hipStream_t s = (hipStream_t)stream;
+    {
+        mkv::ProfScope prof(MKV_K_FILL_ZERO, s);
+        hipLaunchKernelGGL(mkv::fill_zero_kernel, dim3((unsigned)want), dim3(256), 0, s, (uint4*)ptr,
+                           units, (uint8_t*)ptr + (units << 4), tail);
+    }
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_swap_blocks(const int64_t* src_ids, const int64_t* dst_ids, int64_t count,
+                    int32_t is_swap_in, const mkv_pool* pool, void* k_swap, void* v_swap,
+                    int64_t* num_copies, void* stream) {
+    int rc = mkv::check_pool(pool);
+    if (rc) return rc;
+    MKV_REQUIRE(count >= 0, "count must be >= 0");
+    if (num_copies) *num_copies = 0;
+    if (count == 0) return MKV_OK;
+    MKV_REQUIRE(src_ids && dst_ids && k_swap && v_swap, "NULL argument");
+    const int64_t block_bytes = mkv::pool_block_bytes(*pool);
+    const int64_t total_blocks = mkv::pool_total_blocks(*pool);
+    // the device side of the pair: target on swap-in, source on swap-out
+    const int64_t* dev_ids = is_swap_in ? dst_ids : src_ids;
+    const int64_t* host_ids = is_swap_in ? src_ids : dst_ids;
+    auto seg_of = [&](int64_t id) -> int64_t {
+        return id < pool->num_blocks_org ? -1 : (id - pool->num_blocks_org) / pool->seg_blocks;
+    };
+    for (int64_t i = 0; i < count; ++i) {
+        MKV_REQUIRE(dev_ids[i] >= 0 && dev_ids[i] < total_blocks,
+                    "device block id %lld outside the pool (%lld blocks)", (long long)dev_ids[i],
+                    (long long)total_blocks);
+        MKV_REQUIRE(host_ids[i] >= 0, "host block id %lld is negative", (long long)host_ids[i]);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    int64_t copies = 0;
+    int64_t i = 0;
+    while (i < count) {
+        int64_t j = i + 1;
+        const int64_t seg = seg_of(dev_ids[i]);
+        while (j < count && src_ids[j] == src_ids[j - 1] + 1 && dst_ids[j] == dst_ids[j - 1] + 1 &&
+               seg_of(dev_ids[j]) == seg)
+            ++j;
+        const int64_t bytes = (j - i) * block_bytes;
+        const int64_t id = dev_ids[i];
+        char *kd, *vd;
+        if (seg < 0) {
+            kd = (char*)pool->k_base + id * block_bytes;
+            vd = (char*)pool->v_base + id * block_bytes;
+        } else {
+            const int64_t local = id - pool->num_blocks_org - seg * pool->seg_blocks;
+            kd = (char*)pool->k_seg[seg] + local * block_bytes;
+            vd = (char*)pool->v_seg[seg] + local * block_bytes;
+        }
+        char* kh = (char*)k_swap + host_ids[i] * block_bytes;
+        char* vh = (char*)v_swap + host_ids[i] * block_bytes;
+        if (is_swap_in) {
+            MKV_HIP(hipMemcpyAsync(kd, kh, bytes, hipMemcpyHostToDevice, s));
+            MKV_HIP(hipMemcpyAsync(vd, vh, bytes, hipMemcpyHostToDevice, s));
+        } else {
+            MKV_HIP(hipMemcpyAsync(kh, kd, bytes, hipMemcpyDeviceToHost, s));
+            MKV_HIP(hipMemcpyAsync(vh, vd, bytes, hipMemcpyDeviceToHost, s));
+        }
+        ++copies;
+        i = j;
+    }
+    if (num_copies) *num_copies = copies;
+    return MKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+"""``paged_attention``: decode attention over the paged cache.
+
+Operator surface of MorphServe/worker/kernels/paged_attn.py:700-1015 (phase 1
+:59-240 / :243-437, phase 2 :658-696) on top of ``mkv_paged_attn_decode``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ... import _capi
+from ._pool import pool_from_args
+
+# Scratch for the per-split partials, grown on demand and reused across calls
+# (the reference allocates it on every call, paged_attn.py:780-793).
+_scratch: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+
+# "auto": split length chosen here for the MI355X grid; "reference": use the
+# caller's infer_state.seq_block_size as the reference kernels do.
+SPLIT_POLICY = os.environ.get("MORPHKV_SPLIT_POLICY", "auto")
+TARGET_WORKGROUPS = int(os.environ.get("MORPHKV_TARGET_WGS", "1536"))
+
+
+def choose_split(n: int, num_kv_heads: int, max_len: int, block_size: int,
+                 target_wgs: Optional[int] = None) -> Tuple[int, int]:
+    """``(tokens_per_split, max_splits)``: enough (split, kv head, sequence)
+    workgroups to cover the 256 compute units several times over, each split a
+    multiple of four blocks (one per wave) and never shorter than 128 tokens."""
+    target = TARGET_WORKGROUPS if target_wgs is None else target_wgs
+    unit = 4 * block_size
+    max_len = max(int(max_len), 1)
+    want = max(1, -(-target // max(1, n * num_kv_heads)))
+    most = max(1, max_len // (2 * unit))
+    splits = min(want, most)
+    tps = -(-max_len // splits)
+    tps = -(-tps // unit) * unit
+    return tps, -(-max_len // tps)
+
+
+def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
+    need_lse = n * hq * splits
+    key = (device.index or 0, d)
+    cur = _scratch.get(key)
+    if cur is None or cur[1].numel() < need_lse:
+        grow = max(need_lse, 2 * cur[1].numel() if cur else 0)
+        cur = (torch.empty(grow * d, dtype=torch.float32, device=device),
+               torch.empty(grow, dtype=torch.float32, device=device))
+        _scratch[key] = cur
+    return cur
+
+
+def paged_attention(
+    q: torch.Tensor,                    # [num_decoding_seqs, num_q_heads, head_dim]
+    k_cache: torch.Tensor,              # [num_blocks, num_layers, num_kv_heads, block_size, head_dim]
+    v_cache: torch.Tensor,
+    k_cache_new: List[torch.Tensor],
+    v_cache_new: List[torch.Tensor],
+    block_table: torch.Tensor,          # [max_seqs, max_blocks_per_seq] int32
+    model_config,
+    engine_config,
+    infer_state,
+    cur_layer: int,
+    o: torch.Tensor,                    # [num_decoding_seqs, num_q_heads*head_dim] (or 3-D), written
+) -> None:
+    assert q.is_contiguous()
+    assert k_cache.is_contiguous()
+    assert v_cache.is_contiguous()
+    assert block_table.is_contiguous()
+    assert infer_state.seq_block_size % engine_config.block_size == 0
+    assert o.is_contiguous()
+    assert q.dtype == torch.float16 and o.dtype == torch.float16
+
+    n = infer_state.num_decoding_seqs
+    if n == 0:
+        return
+    hq = model_config.num_q_heads
+    d = model_config.head_dim
+    block_size = engine_config.block_size
+
+    max_len = infer_state.num_seq_blocks * infer_state.seq_block_size
+    known = getattr(infer_state, "max_decoding_len", 0)
+    if known:
+        max_len = min(max_len, int(known)) if max_len > 0 else int(known)
+    if SPLIT_POLICY == "reference":
+        tps, splits = infer_state.seq_block_size, max(1, infer_state.num_seq_blocks)
+    else:
+        tps, splits = choose_split(n, model_config.num_kv_heads, max_len, block_size)
+
+    lib = _capi.lib()
+    pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
+    mid_o, mid_lse = (None, None)
+    if splits > 1:
+        mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
+    ids_off = infer_state.num_prefill_seqs * infer_state.seq_ids.element_size()
+    _capi.check(lib.mkv_paged_attn_decode(
+        q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
+        infer_state.seq_ids.data_ptr() + ids_off, infer_state.decoding_seq_lens.data_ptr(),
+        n, hq, float(infer_state.softmax_scale), cur_layer, tps, splits,
+        _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))

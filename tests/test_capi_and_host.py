@@ -1,0 +1,110 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header
+declares (no compute calls here), and the host-side logic of the operator mirror."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "morphkv.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = _declared()
+    for must in ("mkv_append_decode", "mkv_append_prefill", "mkv_paged_attn_decode", "mkv_prefill_attn",
+                 "mkv_bm_allocate", "mkv_bt_append", "mkv_bt_release", "mkv_bt_gather_release",
+                 "mkv_pool_plan_shrink", "mkv_pool_migrate", "mkv_bt_remap", "mkv_swap_blocks",
+                 "mkv_pool_carve_segment", "mkv_fill_zero"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from morphserve_amd import _capi
+    lib = _capi.lib()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} is declared in morphkv.h but not exported"
+        assert name in _capi.PROTOTYPES, f"{name} has no ctypes prototype"
+    assert lib.mkv_version() >= 1
+    assert ctypes.sizeof(_capi.MkvPool) == lib.mkv_sizeof_pool() == 56 + 2 * 8 * _capi.MKV_MAX_SEGMENTS
+
+
+def test_host_only_entry_points():
+    """Entry points that do no GPU work can be exercised without a GPU."""
+    from morphserve_amd import _capi, swiftllm_c
+    lib = _capi.lib()
+    k0, s, v0 = ctypes.c_uint64(0), ctypes.c_int64(0), ctypes.c_uint64(0)
+    rc = lib.mkv_pool_carve_segment(1000, 4000, 300, 2, 2, 4, 8, ctypes.byref(k0), ctypes.byref(s), ctypes.byref(v0))
+    assert rc == 0 and (k0.value, s.value, v0.value) == R.acquire_new_kvcache_arith(1000, 4000, 300, 2, 2, 4, 8)
+    rc = lib.mkv_pool_carve_segment(0, 1000, 600, 2, 2, 4, 8, ctypes.byref(k0), ctypes.byref(s), ctypes.byref(v0))
+    assert rc == _capi.MKV_ENOSPC and b"No space available" in lib.mkv_last_error()
+    MiB = 1 << 20
+    swiftllm_c.register_kv_cache_info(32, 8, 16, 128)
+    assert swiftllm_c.carve_segment(7 * MiB, 436 * MiB, 120 * MiB + 5) == \
+        R.acquire_new_kvcache_arith(7 * MiB, 436 * MiB, 120 * MiB + 5, 32, 8, 16, 128)
+    # strided segment table: segment j sits j * stride * elem_bytes below segment 0
+    pool = _capi.MkvPool()
+    _capi.check(lib.mkv_pool_set_strided(ctypes.byref(pool), 1 << 30, (1 << 30) + 4096, 1000, 2, 3))
+    assert [pool.k_seg[j] for j in range(3)] == [(1 << 30) - j * 2000 for j in range(3)]
+    assert [pool.v_seg[j] for j in range(3)] == [(1 << 30) + 4096 - j * 2000 for j in range(3)]
+    assert pool.num_segments == 3 and pool.k_seg[3] is None
+    with pytest.raises(_capi.MorphKVError):
+        _capi.check(lib.mkv_pool_set_strided(ctypes.byref(pool), 0, 0, 1000, 2, 999))
+    # argument validation happens before any launch
+    assert lib.mkv_append_decode(None, None, None, None, 0, None, None, 1, 0, None) == _capi.MKV_EINVAL
+    with pytest.raises(NotImplementedError):
+        swiftllm_c.replace_layer_org2quant(0)
+
+
+def test_seq_block_size_matches_oracle():
+    from morphserve_amd import select_seq_block_size
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        n = int(rng.integers(0, 200))
+        lens = rng.integers(1, 5000, size=n).tolist()
+        hkv = int(rng.choice([1, 2, 4, 8, 32]))
+        assert select_seq_block_size(hkv, lens) == R.select_seq_block_size(hkv, lens)
+    assert select_seq_block_size(32, [64, 100, 200, 288, 300, 400, 445, 512]) == (64, 8)
+    assert select_seq_block_size(8, [1280] * 64) == (512, 3)
+
+
+def test_choose_split_properties():
+    from morphserve_amd.worker.kernels.paged_attn import choose_split
+    rng = np.random.default_rng(1)
+    for _ in range(500):
+        n = int(rng.integers(1, 600))
+        hkv = int(rng.choice([1, 2, 4, 8, 32]))
+        max_len = int(rng.integers(1, 40000))
+        tps, splits = choose_split(n, hkv, max_len, 16, target_wgs=int(rng.integers(1, 5000)))
+        assert tps % 64 == 0 and tps > 0
+        assert splits >= 1 and splits * tps >= max_len and (splits - 1) * tps < max_len
+    assert choose_split(64, 8, 1536, 16, target_wgs=1536) == (512, 3)
+    assert choose_split(1000, 32, 512, 16, target_wgs=1536) == (512, 1)
+
+
+def test_block_count_behaves_like_the_reference_counter():
+    from morphserve_amd.worker.block_manager import BlockCount
+    c = BlockCount(10)
+    c -= 3
+    c += 2
+    assert c == 9 and c.item() == 9 and isinstance(c, int) and isinstance(c + 1, BlockCount)
+    assert (c >= 9) and (100 - c == 91) and f"{c}" == "9"
+
+
+def test_product_does_not_import_the_oracle():
+    """The shipped package must never reach into the test oracle."""
+    pkg = os.path.join(ROOT, "morphserve_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
