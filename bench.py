@@ -1,0 +1,337 @@
+"""Benchmark of the paged-KV hot path on one MI355X.
+
+Default workload (``cfg2_llama3_8b_decode``): Llama-3-8B-shaped decode -- 32
+layers, GQA 32 q / 8 kv heads, head_dim 128, block_size 16, batch 64, contexts
+uniform in [1024, 1536], KV pool of 65 536 blocks (128 GiB) with randomly
+permuted block tables, Q/K/V ~ N(0,1).  One step = for every layer: append one
+token per sequence to the paged cache, then paged decode attention.
+
+Prints ONE JSON line: whole-step throughput in algorithmic HBM GB/s (inputs
+resident in HBM), the roofline of the dominant kernel (decode attention phase 1,
+timed per launch with HIP events on its own stream) and a CPU baseline (the
+oracle's torch-CPU statement of the same path on a bounded sample).
+
+``--workload cfg3_resize`` measures the elastic pool instead: grow 32k -> 96k
+blocks (zero fill), scatter ~24.5k live blocks, shrink to 40k with migration.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+
+
+class Cfg:
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
+                    choices=["cfg2_llama3_8b_decode", "cfg3_resize"])
+    ap.add_argument("--pool-blocks", type=int, default=65536)
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=2)
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------------
+def decode_bytes_per_layer(lens, n, hq, hkv, d, b):
+    """Algorithmic HBM bytes of one layer: every K/V slab once, q, o, table; plus the append."""
+    lens = np.asarray(lens, dtype=np.int64)
+    attn = int(lens.sum()) * 2 * hkv * d * 2 + 2 * n * hq * d * 2 + int(((lens + b - 1) // b).sum()) * 4
+    append = 2 * (n * 2 * hkv * d * 2)            # read k, v rows + write them into the cache
+    return attn, append
+
+
+def bench_decode(args):
+    import torch
+    from morphserve_amd import _capi, build_infer_state, paged_attention, store_kvcache
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(1024, 1537, size=N).astype(np.int32)
+    nblk = (lens.astype(np.int64) + B - 1) // B
+    num_blocks = args.pool_blocks
+    max_blocks_per_seq = 128
+    max_seqs = 256
+
+    # block tables: a seeded permutation of the whole pool dealt in order
+    perm = rng.permutation(num_blocks)
+    seq_ids = rng.permutation(max_seqs)[:N].astype(np.int32)
+    table = np.full((max_seqs, max_blocks_per_seq), -1, dtype=np.int32)
+    pos = 0
+    for i in range(N):
+        table[seq_ids[i], :nblk[i]] = perm[pos:pos + nblk[i]]
+        pos += nblk[i]
+    live = perm[:pos].copy()
+
+    shape = (num_blocks, L, HKV, B, D)
+    k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+    v_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    live_t = torch.from_numpy(live).to(dev)
+    for c0 in range(0, len(live), 256):           # N(0,1) in the live blocks, 256 blocks at a time
+        idx = live_t[c0:c0 + 256]
+        k_cache[idx] = torch.randn((len(idx), *shape[1:]), dtype=torch.float16, device=dev, generator=g)
+        v_cache[idx] = torch.randn((len(idx), *shape[1:]), dtype=torch.float16, device=dev, generator=g)
+    bt = torch.from_numpy(table).to(dev)
+    q = torch.randn((L, N, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    k_new = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    v_new = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((L, N, HQ * D), dtype=torch.float16, device=dev)
+
+    model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
+    engine = Cfg(block_size=B, max_blocks_per_seq=max_blocks_per_seq)
+    st = build_infer_state([], seq_ids.tolist(), lens.tolist(), HKV, D)
+
+    def step():
+        for layer in range(L):
+            store_kvcache(k_new[layer], v_new[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer)
+            paged_attention(q[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer, o[layer])
+
+    # -- warmup, then the timed region --------------------------------------------------
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+    run = graph.replay if graph is not None else step
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # eager step time too (CPU launch overhead included), for the record
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(3, args.steps // 4)):
+        step()
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / max(3, args.steps // 4)
+
+    # -- dominant kernel: per-launch duration with HIP events on its stream -------------
+    _capi.prof_reset()
+    _capi.prof_enable(True)
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    launches, total_ms = _capi.prof_collect(_capi.K_ATTN_PHASE1)
+    p2_launches, p2_ms = _capi.prof_collect(_capi.K_ATTN_PHASE2)
+    ap_launches, ap_ms = _capi.prof_collect(_capi.K_APPEND_DECODE)
+    _capi.prof_enable(False)
+    _capi.prof_reset()
+    phase1_ms = total_ms / max(launches, 1)
+
+    attn_bytes, append_bytes = decode_bytes_per_layer(lens, N, HQ, HKV, D, B)
+    step_bytes = (attn_bytes + append_bytes) * L
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = attn_bytes / (phase1_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "paged decode-attn+KV-append HBM GB/s (% of peak) and decode tokens/s, 1 MI355X",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": "cfg2_llama3_8b_decode: 32 layers, GQA 32q/8kv, head_dim 128, block 16, "
+                               f"batch 64, ctx U[1024,1536], pool {num_blocks} blocks "
+                               f"({num_blocks * 2 // 1024} GiB), permuted tables",
+                   "timed_as": "eager launches" if graph is None else "HIP graph replay of one step (96 kernel launches)"},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "eager_ms_per_step": round(eager_ms, 4),
+        "step_algorithmic_bytes": step_bytes,
+        "roofline": {"bound": "hbm", "kernel": "attn_decode_phase1<4>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
+                     "algorithmic_bytes_per_launch": attn_bytes,
+                     "phase2_avg_ms": round(p2_ms / max(p2_launches, 1), 5),
+                     "append_avg_ms": round(ap_ms / max(ap_launches, 1), 5)},
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, v_new,
+                                                  HQ, HKV, D, B, attn_bytes + append_bytes)
+    return out
+
+
+def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, v_new, HQ, HKV, D, B,
+                        bytes_per_layer):
+    """The oracle's torch-CPU path (append + paged attention as the reference's own
+    PyTorch statement) on ONE layer of the same batch; the pool on the host holds
+    only the live blocks, renumbered."""
+    import torch
+    from oracle import ref_cpu as R
+
+    layer = 0
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    live_sorted = np.sort(live)
+    renum = {int(b): j for j, b in enumerate(live_sorted)}
+    idx = torch.from_numpy(live_sorted).to(k_cache.device)
+    kl = k_cache[idx, layer].cpu().numpy()          # [nlive, Hkv, B, D]
+    vl = v_cache[idx, layer].cpu().numpy()
+    nlive = len(live_sorted)
+    lay = R.plain_layout(nlive, 1, HKV, B, D)
+    arena = np.concatenate([kl.reshape(-1), vl.reshape(-1)])
+    t2 = table.copy()
+    for s in seq_ids:
+        row = t2[s]
+        for j in range(len(row)):
+            if row[j] >= 0:
+                row[j] = renum[int(row[j])]
+    qh = q[layer].cpu().numpy()
+    kh = k_new[layer].cpu().numpy()
+    vh = v_new[layer].cpu().numpy()
+    reps, t_total = 0, 0.0
+    while t_total < 10.0 and reps < 8:
+        t0 = time.perf_counter()
+        R.append_decode(arena, lay, kh, vh, t2, seq_ids, lens, 0)
+        R.paged_attention(qh, arena, lay, t2, seq_ids, lens, D ** -0.5, 0)
+        t_total += time.perf_counter() - t0
+        reps += 1
+    per_layer = t_total / reps
+    return {"value": round(bytes_per_layer / per_layer / 1e9, 3), "unit": "GB/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of 32 layers of the same batch (64 seqs, ctx 1024-1536), {reps} repetitions, "
+                      f"{per_layer * 1e3:.1f} ms per layer; x32 layers = {per_layer * 32 * 1e3:.0f} ms per step (extrapolated)",
+            "host_cpu_count": os.cpu_count()}
+
+
+# ---------------------------------------------------------------------------------
+def bench_resize(args):
+    import torch
+    from morphserve_amd import ElasticKVPool, _capi
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, HKV, D, B = 32, 8, 128, 16
+    ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1          # 32k -> 96k -> 40k blocks of 2 MiB
+    rng = np.random.default_rng(args.seed)
+    pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256)
+    blk_bytes = pool.block_bytes
+    _capi.prof_reset()
+    _capi.prof_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(NSEG):
+        pool.expand(SEG)
+    torch.cuda.synchronize()
+    expand_s = time.perf_counter() - t0
+    fz_launches, fz_ms = _capi.prof_collect(_capi.K_FILL_ZERO)
+    grown = NSEG * SEG
+    fill_gbs = grown * 2 * blk_bytes / (fz_ms * 1e-3) / 1e9
+
+    total = ORG + grown
+    new_n = ORG + KEEP * SEG
+    n_live = int(0.6 * new_n)                          # 24 576 live blocks scattered over the 96k range
+    live = rng.permutation(total)[:n_live]
+    bm = pool.block_manager
+    per_seq = 192
+    n_seq = n_live // per_seq
+    table = np.full((512, 256), -1, dtype=np.int32)
+    n_alloc = np.zeros(512, dtype=np.int32)
+    for s in range(n_seq):
+        table[s, :per_seq] = live[s * per_seq:(s + 1) * per_seq]
+        n_alloc[s] = per_seq
+    live = live[:n_seq * per_seq]
+    free = np.ones(total, dtype=bool)
+    free[live] = False
+    bm.block_table.copy_(torch.from_numpy(table))
+    bm.num_seq_allocated_blocks.copy_(torch.from_numpy(n_alloc))
+    bm.is_block_free.copy_(torch.from_numpy(free))
+    bm.num_free_blocks = int(free.sum())
+    moves_expected = int((live >= new_n).sum())
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    src, dst = pool.shrink_to(new_n)
+    torch.cuda.synchronize()
+    shrink_s = time.perf_counter() - t0
+    mg_launches, mg_ms = _capi.prof_collect(_capi.K_MIGRATE)
+    _capi.prof_enable(False)
+    _capi.prof_reset()
+    moves = int(src.numel())
+    assert moves == moves_expected
+    moved_bytes = moves * 2 * blk_bytes
+    traffic = 2 * moved_bytes                          # read + write
+    achieved = traffic / (mg_ms * 1e-3) / 1e9
+    whole = traffic / shrink_s / 1e9
+    return {
+        "metric": "pool resize + live-block migration HBM GB/s (read+write), 1 MI355X",
+        "value": round(whole, 1), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 0,
+        "ms_per_step": round(shrink_s * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"cfg3_resize: 2 MiB blocks (32 layers x 8 kv heads x 16 x 128 fp16, K+V), "
+                               f"grow {ORG}->{total} (zero fill), {len(live)} live scattered, shrink to {new_n}"},
+        "moves": moves, "moved_GiB": round(moved_bytes / 2 ** 30, 2),
+        "expand_s": round(expand_s, 4), "zero_fill_GBs": round(fill_gbs, 1),
+        "pct_of_hbm_peak": round(100 * whole / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_launch_ms": round(mg_ms / max(mg_launches, 1), 4),
+                     "algorithmic_bytes_per_launch": traffic},
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's throughput; this build uses a single GPU "
+              f"(--gpus {args.gpus} is not supported)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from morphserve_amd import _capi
+    _capi.lib()
+    out = bench_decode(args) if args.workload == "cfg2_llama3_8b_decode" else bench_resize(args)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

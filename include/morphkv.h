@@ -138,8 +138,9 @@ int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
  * sum(need) lowest free ids ascending are marked used, written to new_ids
  * (int64, capacity new_ids_cap) and appended to the table rows in batch order.
  * result (3 x int64, device) receives {total_need, status, free_found}; status
- * 0 ok, MKV_ELOGIC if some need_i < 0 (or a seq id / row length is out of
- * range), MKV_ENOSPC if fewer than total_need
+ * 0 ok, MKV_ELOGIC if some need_i < 0, MKV_EINVAL if a seq id is outside
+ * [0, max_seqs) or a target needs more than max_blocks_per_seq blocks,
+ * MKV_ENOSPC if fewer than total_need
  * blocks are free or total_need > new_ids_cap; on a non-zero status no state
  * is modified. */
 int mkv_bm_allocate(int32_t* num_seq_allocated_blocks, int64_t max_seqs,

@@ -115,17 +115,18 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
     for (int i = tid; i < batch; i += kScanThreads) {
         const int64_t target = ((int64_t)target_lens[i] + block_size - 1) / block_size;
         const int64_t seq = seq_ids[i];
-        if (seq < 0 || seq >= max_seqs) { s_bad = 1; continue; }
+        if (seq < 0 || seq >= max_seqs) { s_bad = 2; continue; }
         const int64_t have = n_alloc[seq];
         const int64_t need = target - have;
-        if (need < 0 || target > max_blocks_per_seq) s_bad = 1;
+        if (target > max_blocks_per_seq) s_bad = 2;       // would not fit the table row
+        else if (need < 0) atomicMax(&s_bad, 1);
         my_need += need;
     }
     int64_t total;
     block_excl_scan(my_need, &total, sm);
     __syncthreads();
     if (s_bad) {
-        if (tid == 0) { result[0] = total; result[1] = MKV_ELOGIC; result[2] = 0; }
+        if (tid == 0) { result[0] = total; result[1] = (s_bad == 2) ? MKV_EINVAL : MKV_ELOGIC; result[2] = 0; }
         return;
     }
     if (total == 0) {

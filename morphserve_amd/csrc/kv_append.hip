@@ -28,6 +28,7 @@ __global__ __launch_bounds__(256) void append_decode_kernel(
     const int pos = seq_lens[i] - 1;
     const int blk = pos / pool.block_size;
     const int off = pos - blk * pool.block_size;
+    if (pos < 0 || blk >= max_blocks_per_seq) return;        // no such position in the table row
     const int64_t pid = block_table[seq * max_blocks_per_seq + blk];
     if (pid < 0 || pid >= pool_total_blocks(pool)) return;   // unallocated row: nothing to write
 

@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const int Hq = pool.num_kv_heads * G;
 
     const int len = seq_lens[i];
-    const int nblk = (len + kB - 1) / kB;
+    const int nblk = (int)min((int64_t)((len + kB - 1) / kB), max_blocks_per_seq);   // never read past the table row
     const int blk_begin = split * blocks_per_split;
     if (blk_begin >= nblk) return;                      // uniform over the workgroup
     // the last launched split also takes whatever lies beyond it, so an

@@ -106,6 +106,9 @@ class BlockManager:
             seq_ids.data_ptr(), target_lens.data_ptr(), batch, self.block_size,
             new_ids.data_ptr(), new_ids.shape[0], self._result.data_ptr(), _capi.current_stream()))
         total, status, found = self._result[:3].tolist()
+        if status == _capi.MKV_EINVAL:
+            raise ValueError(f"(On {self.device_name}) a sequence id is outside the block table or a target "
+                             f"length needs more than {self.block_table.shape[1]} blocks per sequence")
         assert status != _capi.MKV_ELOGIC, \
             f"(On {self.device_name}) Logic error: Some sequences have more blocks already allocated than needed. seq_ids: {seq_ids}, target_lens: {target_lens}"
         if status == _capi.MKV_ENOSPC or total > self.num_free_blocks:

@@ -19,8 +19,8 @@ def _i32(x, dev):
 
 
 def test_hand_scenario(cuda):
-    bm = BlockManager("GPU", 10, 4, 6, 16)
-    ob = R.BlockManagerOracle("GPU", 10, 4, 6, 16)
+    bm = BlockManager("GPU", 10, 4, 12, 16)
+    ob = R.BlockManagerOracle("GPU", 10, 4, 12, 16)
     for ids, lens in (([2, 0], [33, 16]), ([0, 2], [17, 48]), ([0], [32])):
         got = bm.allocate_blocks_for_seqs(_i32(ids, cuda), _i32(lens, cuda))
         want = ob.allocate_blocks_for_seqs(ids, lens)
@@ -41,8 +41,14 @@ def test_hand_scenario(cuda):
         bm.allocate_blocks_for_seqs(_i32([3], cuda), _i32([16 * 11], cuda))
     assert_state_equal(manager_state(bm), before, "failed allocation must not change state")
     bm.allocate_blocks_for_seqs(_i32([3], cuda), _i32([64], cuda))
+    ob.allocate_blocks_for_seqs([3], [64])
     with pytest.raises(AssertionError):
         bm.allocate_blocks_for_seqs(_i32([3], cuda), _i32([16], cuda))
+    with pytest.raises(ValueError):
+        bm.allocate_blocks_for_seqs(_i32([2], cuda), _i32([16 * 13], cuda))      # more than a table row holds
+    with pytest.raises(ValueError):
+        bm.allocate_blocks_for_seqs(_i32([4], cuda), _i32([16], cuda))           # no such sequence slot
+    assert_state_equal(manager_state(bm), ob.snapshot() | {"num_free_blocks": int(bm.num_free_blocks)}, "rejected calls")
     empty = bm.allocate_blocks_for_seqs(_i32([], cuda), _i32([], cuda))
     assert empty.numel() == 0 and empty.dtype == torch.int64
 
@@ -221,7 +227,9 @@ def test_expand_shrink_round_trip(cuda):
     assert_state_equal(manager_state(bm), ob.snapshot(), "expanded")
     assert bm.num_blocks_org == 8 and float(pool.k_cache_new[1].abs().sum()) == 0.0
     assert pool.shrink_tail_if_unused() and pool.shrink_tail_if_unused()
+    assert ob.shrink(4, 2) and ob.shrink(4, 1)
     assert_state_equal(manager_state(bm), snap, "round trip")
+    assert_state_equal(manager_state(bm), ob.snapshot(), "round trip vs oracle")
     pool.expand(4)
     pool.expand(4)
     ob.expand(4)
