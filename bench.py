@@ -45,6 +45,9 @@ def parse_args():
                     choices=["cfg2_llama3_8b_decode", "cfg3_resize"])
     ap.add_argument("--pool-blocks", type=int, default=65536)
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--unfused", action="store_true",
+                    help="time store_kvcache + paged_attention as two calls per layer (default: the fused "
+                         "one-launch-per-layer call)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=2)
     return ap.parse_args()
@@ -61,7 +64,8 @@ def decode_bytes_per_layer(lens, n, hq, hkv, d, b):
 
 def bench_decode(args):
     import torch
-    from morphserve_amd import _capi, build_infer_state, paged_attention, store_kvcache
+    from morphserve_amd import (_capi, build_infer_state, decode_append_and_attend, paged_attention,
+                                store_kvcache)
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -103,10 +107,18 @@ def bench_decode(args):
     engine = Cfg(block_size=B, max_blocks_per_seq=max_blocks_per_seq)
     st = build_infer_state([], seq_ids.tolist(), lens.tolist(), HKV, D)
 
-    def step():
+    def step_two_calls():
         for layer in range(L):
             store_kvcache(k_new[layer], v_new[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer)
             paged_attention(q[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer, o[layer])
+
+    def step_fused():
+        for layer in range(L):
+            decode_append_and_attend(k_new[layer], v_new[layer], q[layer], k_cache, v_cache, [], [], bt,
+                                     model, engine, st, layer, o[layer])
+
+    step = step_two_calls if args.unfused else step_fused
+    other = step_fused if args.unfused else step_two_calls
 
     # -- warmup, then the timed region --------------------------------------------------
     for _ in range(max(args.warmup, 1)):
@@ -137,13 +149,21 @@ def bench_decode(args):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # eager step time too (CPU launch overhead included), for the record
+    # eager step time too (CPU launch overhead included), and the other call shape, for the record
+    reps = max(3, args.steps // 4)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(max(3, args.steps // 4)):
+    for _ in range(reps):
         step()
     torch.cuda.synchronize()
-    eager_ms = (time.perf_counter() - t0) * 1e3 / max(3, args.steps // 4)
+    eager_ms = (time.perf_counter() - t0) * 1e3 / reps
+    other()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        other()
+    torch.cuda.synchronize()
+    other_ms = (time.perf_counter() - t0) * 1e3 / reps
 
     # -- dominant kernel: per-launch duration with HIP events on its stream -------------
     _capi.prof_reset()
@@ -179,17 +199,20 @@ def bench_decode(args):
         "config": {"workload": "cfg2_llama3_8b_decode: 32 layers, GQA 32q/8kv, head_dim 128, block 16, "
                                f"batch 64, ctx U[1024,1536], pool {num_blocks} blocks "
                                f"({num_blocks * 2 // 1024} GiB), permuted tables",
-                   "timed_as": "eager launches" if graph is None else "HIP graph replay of one step (96 kernel launches)"},
+                   "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
+                                      else "decode_append_and_attend (1 fused launch)",
+                   "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
         "eager_ms_per_step": round(eager_ms, 4),
+        ("fused_eager_ms_per_step" if args.unfused else "two_call_eager_ms_per_step"): round(other_ms, 4),
         "step_algorithmic_bytes": step_bytes,
-        "roofline": {"bound": "hbm", "kernel": "attn_decode_phase1<4>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "attn_decode_phase1_mfma<4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None, "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
                      "algorithmic_bytes_per_launch": attn_bytes,
-                     "phase2_avg_ms": round(p2_ms / max(p2_launches, 1), 5),
-                     "append_avg_ms": round(ap_ms / max(ap_launches, 1), 5)},
+                     "phase2_avg_ms": round(p2_ms / max(p2_launches, 1), 5) if p2_launches else None,
+                     "append_avg_ms": round(ap_ms / max(ap_launches, 1), 5) if ap_launches else None},
     }
 
     if not args.no_cpu_baseline:

@@ -107,6 +107,24 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
                           int32_t layer, int32_t tokens_per_split, int32_t max_splits,
                           void* mid_o, void* mid_lse, void* stream);
 
+/* store_kvcache (decode rows) + paged_attention of one layer in ONE launch: the
+ * call pair of MS/worker/layers/transformer_layer.py:116-126, :181-187 for a
+ * decode batch.  k, v : [n, Hkv, D] fp16 is token seq_lens[i]-1 of each
+ * sequence; it is written to its cache slot exactly as mkv_append_decode would
+ * and takes part in the attention from registers.  Other arguments as
+ * mkv_paged_attn_decode. */
+int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,
+                           const mkv_pool* pool, const int32_t* block_table,
+                           int64_t max_blocks_per_seq, const int32_t* seq_ids,
+                           const int32_t* seq_lens, int32_t n, int32_t num_q_heads,
+                           float softmax_scale, int32_t layer, int32_t tokens_per_split,
+                           int32_t max_splits, void* mid_o, void* mid_lse, void* stream);
+
+/* Tuning knob without a counterpart in the reference: which phase-1 kernel
+ * mkv_paged_attn_decode launches.  0 = by GQA group size (matrix cores when
+ * Hq/Hkv >= 4, vector ALU otherwise), 1 = vector ALU, 2 = matrix cores. */
+int mkv_set_decode_variant(int32_t variant);
+
 /* ---- prefill attention -------------------------------------------------- */
 /* prefill_attention, MS/worker/kernels/prefill_attn.py:9-139, and the live
  * flash_attn_varlen_func call, MS/worker/layers/transformer_layer.py:154-164:

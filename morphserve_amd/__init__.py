@@ -18,7 +18,7 @@ from . import _capi  # noqa: F401
 from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
 from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
-from .worker.kernels.paged_attn import paged_attention  # noqa: F401
+from .worker.kernels.paged_attn import decode_append_and_attend, paged_attention  # noqa: F401
 from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401
 from .elastic_pool import ElasticKVPool  # noqa: F401
 from . import swiftllm_c  # noqa: F401

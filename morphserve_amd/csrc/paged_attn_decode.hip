@@ -48,11 +48,7 @@ __device__ __forceinline__ float dot8(const uint4& a, const uint4& b, float acc)
     return acc;
 }
 
-struct Slab {
-    const uint4* k;
-    const uint4* v;
-    bool ok;
-};
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 template <int G>
 struct RowState {
@@ -111,6 +107,38 @@ __device__ __forceinline__ void consume_block(RowState<G>& st, const uint4 (&q)[
     }
 }
 
+// Final step of a phase-1 workgroup: merge the four waves' (max, sum, accumulator)
+// states held in LDS and store either the finished output (one split launched) or
+// this split's normalised partial and its log2-sum-exp.
+template <int G>
+__device__ __forceinline__ void merge_waves_and_store(const float (&sm_acc)[4][G][kD],
+                                                      const float (&sm_m)[4][G],
+                                                      const float (&sm_l)[4][G], __half* o,
+                                                      float* mid_o, float* mid_lse, int64_t hq0,
+                                                      int split, int max_splits) {
+    const bool direct = gridDim.x == 1;
+    for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
+        const int g = idx / kD;
+        const int d = idx - g * kD;
+        const float m_tot = fmaxf(fmaxf(sm_m[0][g], sm_m[1][g]), fmaxf(sm_m[2][g], sm_m[3][g]));
+        float l_tot = 0.f, a_tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float f = fast_exp2(sm_m[w][g] - m_tot);
+            l_tot += sm_l[w][g] * f;
+            a_tot += sm_acc[w][g][d] * f;
+        }
+        const float val = a_tot / l_tot;
+        const int64_t hq = hq0 + g;
+        if (direct) {
+            o[hq * kD + d] = __float2half(val);
+        } else {
+            mid_o[(hq * max_splits + split) * kD + d] = val;
+            if (d == 0) mid_lse[hq * max_splits + split] = log2f(l_tot) + m_tot;
+        }
+    }
+}
+
 template <int G>
 __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ q,        // [n, Hq, D] fp16
@@ -119,7 +147,9 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     float* __restrict__ mid_lse,        // [n, Hq, max_splits]
     const mkv_pool pool, const int32_t* __restrict__ block_table, int64_t max_blocks_per_seq,
     const int32_t* __restrict__ seq_ids, const int32_t* __restrict__ seq_lens, float scale2,
-    int32_t layer, int32_t blocks_per_split, int32_t max_splits) {
+    int32_t layer, int32_t blocks_per_split, int32_t max_splits,
+    const uint4* __restrict__ k_new,    // [n, Hkv, D] fp16 or NULL: token len-1 to append first
+    const uint4* __restrict__ v_new) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -158,54 +188,96 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
         for (int j = 0; j < 8; ++j) st.acc[g][j] = 0.f;
     }
 
-    // This wave's blocks: blk_begin + wave + 4 * it.  Table entries are fetched
-    // 64 iterations at a time (one per lane) and handed out with readlane.
-    const int my_first = blk_begin + wave;
-    const int n_it = (blk_end - my_first + 3) >> 2;      // may be <= 0
-    auto slab_of = [&](int32_t pid) {
-        Slab s;
-        s.ok = pid >= 0 && pid < total_blocks;
-        BlockAddr a = block_addr(pool, s.ok ? pid : 0, block_bytes);
-        s.k = (const uint4*)(a.k + head_off) + lane;
-        s.v = (const uint4*)(a.v + head_off) + lane;
-        return s;
+    // This wave's blocks: blk_begin + wave + 4 * t.  Table entries are fetched 64
+    // iterations at a time (one per lane) and handed out with readlane.  Only the
+    // sequence's final block can be partial; it is the last of its wave's list and
+    // is handled apart, so the main loop carries no masking and no branches around
+    // its loads: the loads of block t+1 are issued before block t is consumed and
+    // stay in flight behind it.
+    const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
+    const int n_it = max(0, (blk_end - my_first + 3) >> 2);
+    // blocks [0, nblk_full) hold 16 valid tokens and need no special care; with a
+    // fused append the final block always does (it receives the new token)
+    const bool fused = k_new != nullptr;
+    const int nblk_full = fused ? nblk - 1 : len / kB;
+    auto load_block = [&](int32_t pid, uint4 (&kk)[4], uint4 (&vv)[4]) {
+        BlockAddr a = block_addr(pool, pid, block_bytes);
+        const v4u* kp = (const v4u*)(a.k + head_off) + lane;
+        const v4u* vp = (const v4u*)(a.v + head_off) + lane;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) kk[x] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(kp + x * 64));
+#pragma unroll
+        for (int x = 0; x < 4; ++x) vv[x] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(vp + x * 64));
     };
 
     for (int it0 = 0; it0 < n_it; it0 += 64) {
         const int b_lane = my_first + 4 * (it0 + lane);
-        const int32_t tbl = (b_lane < blk_end) ? row[b_lane] : -1;
+        const bool in_range = b_lane < blk_end;
+        const int32_t tbl = in_range ? row[b_lane] : 0;
+        const bool bad = in_range && (tbl < 0 || tbl >= total_blocks);
+        const bool any_bad = __ballot(bad) != 0;          // wave-uniform
         const int cnt = min(64, n_it - it0);
+        const int b_last = my_first + 4 * (it0 + cnt - 1);
+        const int cnt_full = (b_last >= nblk_full) ? cnt - 1 : cnt;
+        auto pid_of = [&](int t) { return __builtin_amdgcn_readlane(tbl, t); };
+        auto tok_of = [&](int t) { return (my_first + 4 * (it0 + t)) * kB; };
 
-        uint4 kc[4], vc[4];
-        Slab cur = slab_of(__builtin_amdgcn_readlane(tbl, 0));
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            kc[x] = cur.ok ? cur.k[x * 64] : make_uint4(0u, 0u, 0u, 0u);
-            vc[x] = cur.ok ? cur.v[x * 64] : make_uint4(0u, 0u, 0u, 0u);
+        if (!any_bad) {
+            if (cnt_full > 0) {
+                uint4 k0[4], v0[4], k1[4], v1[4];
+                load_block(pid_of(0), k0, v0);
+                int t = 0;
+                while (t + 2 < cnt_full) {
+                    load_block(pid_of(t + 1), k1, v1);
+                    consume_block<G, false>(st, qreg, k0, v0, scale2, tok_of(t), len, r);
+                    load_block(pid_of(t + 2), k0, v0);
+                    consume_block<G, false>(st, qreg, k1, v1, scale2, tok_of(t + 1), len, r);
+                    t += 2;
+                }
+                if (t + 1 < cnt_full) {
+                    load_block(pid_of(t + 1), k1, v1);
+                    consume_block<G, false>(st, qreg, k0, v0, scale2, tok_of(t), len, r);
+                    consume_block<G, false>(st, qreg, k1, v1, scale2, tok_of(t + 1), len, r);
+                } else {
+                    consume_block<G, false>(st, qreg, k0, v0, scale2, tok_of(t), len, r);
+                }
+            }
+        } else {
+            // a table entry names no block of the pool: skip such blocks
+            for (int t = 0; t < cnt_full; ++t) {
+                const int32_t pid = pid_of(t);
+                if (pid < 0 || pid >= total_blocks) continue;
+                uint4 k0[4], v0[4];
+                load_block(pid, k0, v0);
+                consume_block<G, false>(st, qreg, k0, v0, scale2, tok_of(t), len, r);
+            }
         }
-        for (int t = 0; t < cnt; ++t) {
-            const int b = my_first + 4 * (it0 + t);
-            uint4 kn[4], vn[4];
-            const bool has_next = (t + 1) < cnt;
-            if (has_next) {
-                Slab nx = slab_of(__builtin_amdgcn_readlane(tbl, t + 1));
+        if (cnt_full < cnt) {                              // the partial final block
+            const int32_t pid = pid_of(cnt - 1);
+            if (pid >= 0 && pid < total_blocks) {
+                uint4 k0[4], v0[4];
+                load_block(pid, k0, v0);
+                if (fused) {
+                    // token len-1: write it into its slot of the cache and use it from
+                    // registers, whatever the slot held before
+                    const int off = (len - 1) & (kB - 1);
+                    const uint4 kn = k_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + (lane & 15)];
+                    const uint4 vn = v_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + (lane & 15)];
+                    if (r == (off & 3)) {
+                        BlockAddr a = block_addr(pool, pid, block_bytes);
+                        const int64_t slot = head_off + (int64_t)off * (kD * 2) + (lane & 15) * 16;
+                        *(uint4*)(const_cast<char*>(a.k) + slot) = kn;
+                        *(uint4*)(const_cast<char*>(a.v) + slot) = vn;
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    kn[x] = nx.ok ? nx.k[x * 64] : make_uint4(0u, 0u, 0u, 0u);
-                    vn[x] = nx.ok ? nx.v[x * 64] : make_uint4(0u, 0u, 0u, 0u);
+                        for (int x = 0; x < 4; ++x) {
+                            if (x == (off >> 2)) {
+                                k0[x] = kn;
+                                v0[x] = vn;
+                            }
+                        }
+                    }
                 }
-            }
-            if (b == nblk - 1) {
-                consume_block<G, true>(st, qreg, kc, vc, scale2, b * kB, len, r);
-            } else {
-                consume_block<G, false>(st, qreg, kc, vc, scale2, b * kB, len, r);
-            }
-            if (has_next) {
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    kc[x] = kn[x];
-                    vc[x] = vn[x];
-                }
+                consume_block<G, true>(st, qreg, k0, v0, scale2, tok_of(cnt - 1), len, r);
             }
         }
     }
@@ -246,28 +318,237 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
         }
     }
     __syncthreads();
+    merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
+                             max_splits);
+}
 
-    const bool direct = gridDim.x == 1;
-    for (int idx = tid; idx < G * kD; idx += 256) {
-        const int g = idx / kD;
-        const int d = idx - g * kD;
-        float m_tot = fmaxf(fmaxf(sm_m[0][g], sm_m[1][g]), fmaxf(sm_m[2][g], sm_m[3][g]));
-        float l_tot = 0.f, a_tot = 0.f;
+// ---- matrix-core variant for GQA groups (G >= 4) -----------------------------------
+// Same workgroup / wave decomposition.  A wave stages each 16-token K and V tile
+// in its private LDS area (row-major, rows padded to 272 bytes) and reads it back
+// in matrix-core operand order:
+//   S^T[token, head] = K[token, :] . Q^T      one v_mfma_f32_16x16x32_f16 per 32 dims,
+//                                             the G heads padded to 16 columns
+//   O^T[dim, head]  += V^T[dim, token] . P^T  one v_mfma_f32_16x16x16_f16 per 16 dims
+// The accumulator layout of S^T (lane = head, registers = four consecutive
+// tokens) is the B-operand layout of the second product, so the probabilities
+// never cross lanes.  Which 8 dims a lane contributes to a product is free as
+// long as K and Q agree, so a lane takes 64 contiguous bytes of its K row.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+static constexpr int kLdsRow = 272;                 // 256 data bytes + 16 pad: conflict-free b128 rows
+static constexpr int kLdsTile = kB * kLdsRow;
+
+struct FullTag { static constexpr bool value = false; };    // a block of 16 valid tokens
+struct FinalTag { static constexpr bool value = true; };    // the sequence's last block: masked
+
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int G>
+__global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
+    const uint4* __restrict__ q, __half* __restrict__ o, float* __restrict__ mid_o,
+    float* __restrict__ mid_lse, const mkv_pool pool, const int32_t* __restrict__ block_table,
+    int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids,
+    const int32_t* __restrict__ seq_lens, float scale2, int32_t layer, int32_t blocks_per_split,
+    int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new) {
+    __shared__ __attribute__((aligned(16))) char stage[4][2][kLdsTile];
+    __shared__ float sm_acc[4][G][kD];
+    __shared__ float sm_m[4][G];
+    __shared__ float sm_l[4][G];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int n = lane & 15;       // head column (B / C operands), token or dim row (A operands)
+    const int c = lane >> 4;       // lane group
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int i = blockIdx.z;
+    const int Hq = pool.num_kv_heads * G;
+
+    const int len = seq_lens[i];
+    const int nblk = (int)min((int64_t)((len + kB - 1) / kB), max_blocks_per_seq);
+    const int blk_begin = split * blocks_per_split;
+    if (blk_begin >= nblk) return;
+    const int blk_end = (split == (int)gridDim.x - 1) ? nblk : min(blk_begin + blocks_per_split, nblk);
+    const int64_t seq = seq_ids[i];
+    const int32_t* row = block_table + seq * max_blocks_per_seq;
+    const int64_t block_bytes = pool_block_bytes(pool);
+    const int64_t total_blocks = pool_total_blocks(pool);
+    const int64_t head_off = ((int64_t)layer * pool.num_kv_heads + kvh) * (kB * kD * 2);
+
+    // Q^T as B operand: lane (head n, group c) holds dims c*32 + 8x .. +8 for product x
+    v8h qb[4];
+    if (n < G) {
+        const uint4* qp = q + ((int64_t)i * Hq + kvh * G + n) * (kD / 8) + c * 4;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float f = fast_exp2(sm_m[w][g] - m_tot);
-            l_tot += sm_l[w][g] * f;
-            a_tot += sm_acc[w][g][d] * f;
+        for (int x = 0; x < 4; ++x) qb[x] = __builtin_bit_cast(v8h, qp[x]);
+    } else {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) qb[x] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+
+    v4f oacc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) oacc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+    float m_run = kNegBig;         // running max of head n (same in the four lane groups)
+    float l_run = 0.f;             // this lane's share of the running sum
+
+    char* kl = stage[wave][0];
+    char* vl = stage[wave][1];
+    const int wr_off = c * kLdsRow + n * 16;                     // load x of lane (c, n): token 4x + c, bytes 16n..
+    const char* k_rd = kl + n * kLdsRow + c * 64;                // token row n, 64 bytes of it
+    const _Float16* v_rd = (const _Float16*)(vl + 4 * c * kLdsRow) + n;   // tokens 4c.., dim n of each tile
+
+    auto issue_loads = [&](int32_t pid, v4u (&kg)[4], v4u (&vg)[4]) {
+        BlockAddr a = block_addr(pool, pid, block_bytes);
+        const v4u* kp = (const v4u*)(a.k + head_off) + lane;
+        const v4u* vp = (const v4u*)(a.v + head_off) + lane;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) kg[x] = __builtin_nontemporal_load(kp + x * 64);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) vg[x] = __builtin_nontemporal_load(vp + x * 64);
+    };
+    // registers -> LDS
+    auto stage_tile = [&](const v4u (&kg)[4], const v4u (&vg)[4]) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            *(v4u*)(kl + wr_off + x * 4 * kLdsRow) = kg[x];
+            *(v4u*)(vl + wr_off + x * 4 * kLdsRow) = vg[x];
         }
-        const float val = a_tot / l_tot;
-        const int64_t hq = (int64_t)i * Hq + kvh * G + g;
-        if (direct) {
-            o[hq * kD + d] = __float2half(val);
+        wave_lds_fence();
+    };
+    // The sequence's final block: rows of tokens at or beyond len are zeroed so that
+    // stale bytes (NaN included) cannot reach either product.
+    auto mask_final_tile = [&](v4u (&kg)[4], v4u (&vg)[4], int tok0) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            if (tok0 + 4 * x + c >= len) {
+                kg[x] = (v4u){0u, 0u, 0u, 0u};
+                vg[x] = (v4u){0u, 0u, 0u, 0u};
+            }
+        }
+    };
+    // Fused append: token len-1 goes into its cache slot and, whatever the slot
+    // held, into the staged tile (one 256-byte row of K and of V, 16 lanes each).
+    auto append_into_tile = [&](int32_t pid) {
+        const int off = (len - 1) & (kB - 1);
+        if (lane < 32) {
+            const bool is_v = lane >= 16;
+            const int64_t src = ((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + n;
+            const v4u val = __builtin_bit_cast(v4u, is_v ? v_new[src] : k_new[src]);
+            BlockAddr a = block_addr(pool, pid, block_bytes);
+            const int64_t slot = head_off + (int64_t)off * (kD * 2) + n * 16;
+            *(v4u*)(const_cast<char*>(is_v ? a.v : a.k) + slot) = val;
+            *(v4u*)((is_v ? vl : kl) + off * kLdsRow + n * 16) = val;
+        }
+        wave_lds_fence();
+    };
+    auto compute_tile = [&](int tok0, auto partial_tag) {
+        constexpr bool partial = decltype(partial_tag)::value;
+        v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const v8h a = *(const v8h*)(k_rd + x * 16);
+            s = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[x], s, 0, 0, 0);
+        }
+        float sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sc[j] = s[j] * scale2;
+            if (partial && tok0 + 4 * c + j >= len) sc[j] = kNegBig;
+        }
+        float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        if (__ballot(m_new > m_run) != 0) {          // some head's max moved: rescale (wave-uniform branch)
+            const float alpha = fast_exp2(m_run - m_new);
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) oacc[t] *= alpha;
+            m_run = m_new;
+        }
+        float p[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) p[j] = fast_exp2(sc[j] - m_run);
+        l_run += (p[0] + p[1]) + (p[2] + p[3]);
+        const v4h pb = (v4h){(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3]};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            v4h va;
+            va[0] = v_rd[0 * (kLdsRow / 2) + 16 * t];
+            va[1] = v_rd[1 * (kLdsRow / 2) + 16 * t];
+            va[2] = v_rd[2 * (kLdsRow / 2) + 16 * t];
+            va[3] = v_rd[3 * (kLdsRow / 2) + 16 * t];
+            oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, pb, oacc[t], 0, 0, 0);
+        }
+        wave_lds_fence();                            // reads done before the next tile is staged
+    };
+
+    const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
+    const int n_it = max(0, (blk_end - my_first + 3) >> 2);
+    // blocks [0, nblk_full) hold 16 valid tokens; the final block takes the careful
+    // path when it is partial or, with a fused append, always
+    const int nblk_full = (k_new != nullptr) ? nblk - 1 : len / kB;
+    for (int it0 = 0; it0 < n_it; it0 += 64) {
+        const int b_lane = my_first + 4 * (it0 + lane);
+        const bool in_range = b_lane < blk_end;
+        const int32_t tbl = in_range ? row[b_lane] : 0;
+        const bool bad = in_range && (tbl < 0 || tbl >= total_blocks);
+        const bool any_bad = __ballot(bad) != 0;
+        const int cnt = min(64, n_it - it0);
+        const int b_last = my_first + 4 * (it0 + cnt - 1);
+        const int cnt_full = (b_last >= nblk_full) ? cnt - 1 : cnt;
+        auto pid_of = [&](int t) { return __builtin_amdgcn_readlane(tbl, t); };
+        auto tok_of = [&](int t) { return (my_first + 4 * (it0 + t)) * kB; };
+        v4u kg[4], vg[4];
+        if (!any_bad) {
+            // block t is staged from registers, block t+1's loads go out, block t is consumed
+            issue_loads(pid_of(0), kg, vg);
+            for (int t = 0; t < cnt_full; ++t) {
+                stage_tile(kg, vg);
+                if (t + 1 < cnt) issue_loads(pid_of(t + 1), kg, vg);
+                compute_tile(tok_of(t), FullTag{});
+            }
+            if (cnt_full < cnt) {
+                mask_final_tile(kg, vg, tok_of(cnt - 1));
+                stage_tile(kg, vg);
+                if (k_new != nullptr && tok_of(cnt - 1) + kB >= len) append_into_tile(pid_of(cnt - 1));
+                compute_tile(tok_of(cnt - 1), FinalTag{});
+            }
         } else {
-            mid_o[(hq * max_splits + split) * kD + d] = val;
-            if (d == 0) mid_lse[hq * max_splits + split] = log2f(l_tot) + m_tot;
+            for (int t = 0; t < cnt; ++t) {
+                const int32_t pid = pid_of(t);
+                if (pid < 0 || pid >= total_blocks) continue;      // names no block of the pool
+                issue_loads(pid, kg, vg);
+                if (t >= cnt_full) mask_final_tile(kg, vg, tok_of(t));
+                stage_tile(kg, vg);
+                if (t >= cnt_full && k_new != nullptr && tok_of(t) + kB >= len) append_into_tile(pid);
+                compute_tile(tok_of(t), FinalTag{});
+            }
         }
     }
+
+    float l_tot = l_run + __shfl_xor(l_run, 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    if (n < G) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sm_acc[wave][n][16 * t + 4 * c + j] = oacc[t][j];
+        if (c == 0) {
+            sm_m[wave][n] = m_run;
+            sm_l[wave][n] = l_tot;
+        }
+    }
+    __syncthreads();
+    merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
+                             max_splits);
 }
 
 // Phase 2: one workgroup of 128 threads per (sequence, q head): log-sum-exp merge
@@ -296,20 +577,39 @@ __global__ __launch_bounds__(128) void attn_decode_phase2(
     o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(ns > 0 ? acc / l : 0.f);
 }
 
+// 0: by group size (matrix cores for G >= 4), 1: vector ALU kernel, 2: matrix-core kernel
+static int g_decode_variant = 0;
+
 template <int G>
 static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void* mid_o,
                           void* mid_lse, const mkv_pool* pool, const int32_t* block_table,
                           int64_t max_blocks_per_seq, const int32_t* seq_ids,
                           const int32_t* seq_lens, float scale2, int32_t layer,
-                          int32_t blocks_per_split, int32_t max_splits) {
-    hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
-                       (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
-                       seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits);
+                          int32_t blocks_per_split, int32_t max_splits, const void* k_new,
+                          const void* v_new) {
+    const bool mfma = g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
+    if (mfma) {
+        hipLaunchKernelGGL(attn_decode_phase1_mfma<G>, grid, dim3(256), 0, s, (const uint4*)q,
+                           (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
+                           max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
+                           max_splits, (const uint4*)k_new, (const uint4*)v_new);
+    } else {
+        hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
+                           (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
+                           seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
+                           (const uint4*)k_new, (const uint4*)v_new);
+    }
 }
 
 }  // namespace mkv
 
 extern "C" {
+
+int mkv_set_decode_variant(int32_t variant) {
+    MKV_REQUIRE(variant >= 0 && variant <= 2, "variant must be 0 (auto), 1 (vector ALU) or 2 (matrix core)");
+    mkv::g_decode_variant = variant;
+    return MKV_OK;
+}
 
 int mkv_paged_attn_scratch_bytes(int32_t n, int32_t num_q_heads, int32_t head_dim,
                                  int32_t max_splits, int64_t* mid_o_bytes,
@@ -321,12 +621,11 @@ int mkv_paged_attn_scratch_bytes(int32_t n, int32_t num_q_heads, int32_t head_di
     return MKV_OK;
 }
 
-int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
-                          const int32_t* block_table, int64_t max_blocks_per_seq,
-                          const int32_t* seq_ids, const int32_t* seq_lens, int32_t n,
-                          int32_t num_q_heads, float softmax_scale, int32_t layer,
-                          int32_t tokens_per_split, int32_t max_splits, void* mid_o,
-                          void* mid_lse, void* stream) {
+static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32_t* block_table,
+                       int64_t max_blocks_per_seq, const int32_t* seq_ids, const int32_t* seq_lens,
+                       int32_t n, int32_t num_q_heads, float softmax_scale, int32_t layer,
+                       int32_t tokens_per_split, int32_t max_splits, void* mid_o, void* mid_lse,
+                       const void* k_new, const void* v_new, void* stream) {
     int rc = mkv::check_pool(pool);
     if (rc) return rc;
     MKV_REQUIRE(n >= 0, "n must be >= 0");
@@ -355,7 +654,7 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
     case GG:                                                                                       \
         mkv::launch_phase1<GG>(grid, s, q, o, mid_o, mid_lse, pool, block_table,                   \
                                max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, bps,          \
-                               max_splits);                                                        \
+                               max_splits, k_new, v_new);                                          \
         break;
             MKV_CASE(1)
             MKV_CASE(2)
@@ -376,6 +675,30 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
         MKV_HIP(hipGetLastError());
     }
     return MKV_OK;
+}
+
+int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
+                          const int32_t* block_table, int64_t max_blocks_per_seq,
+                          const int32_t* seq_ids, const int32_t* seq_lens, int32_t n,
+                          int32_t num_q_heads, float softmax_scale, int32_t layer,
+                          int32_t tokens_per_split, int32_t max_splits, void* mid_o,
+                          void* mid_lse, void* stream) {
+    return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
+                       num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
+                       mid_lse, nullptr, nullptr, stream);
+}
+
+int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,
+                           const mkv_pool* pool, const int32_t* block_table,
+                           int64_t max_blocks_per_seq, const int32_t* seq_ids,
+                           const int32_t* seq_lens, int32_t n, int32_t num_q_heads,
+                           float softmax_scale, int32_t layer, int32_t tokens_per_split,
+                           int32_t max_splits, void* mid_o, void* mid_lse, void* stream) {
+    MKV_REQUIRE(n == 0 || (k && v), "k/v are NULL");
+    MKV_REQUIRE(((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0, "k/v must be 16-byte aligned");
+    return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
+                       num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
+                       mid_lse, k, v, stream);
 }
 
 }  // extern "C"

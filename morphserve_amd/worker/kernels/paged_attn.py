@@ -21,14 +21,16 @@ _scratch: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
 # "auto": split length chosen here for the MI355X grid; "reference": use the
 # caller's infer_state.seq_block_size as the reference kernels do.
 SPLIT_POLICY = os.environ.get("MORPHKV_SPLIT_POLICY", "auto")
-TARGET_WORKGROUPS = int(os.environ.get("MORPHKV_TARGET_WGS", "1536"))
+TARGET_WORKGROUPS = int(os.environ.get("MORPHKV_TARGET_WGS", "512"))
 
 
 def choose_split(n: int, num_kv_heads: int, max_len: int, block_size: int,
                  target_wgs: Optional[int] = None) -> Tuple[int, int]:
     """``(tokens_per_split, max_splits)``: enough (split, kv head, sequence)
-    workgroups to cover the 256 compute units several times over, each split a
-    multiple of four blocks (one per wave) and never shorter than 128 tokens."""
+    workgroups to put two on each of the 256 compute units, and no more: every
+    extra split costs a partial write and the phase-2 launch, and a sequence that
+    is not split at all is written straight to ``o``.  Each split is a multiple
+    of four blocks (one per wave) and never shorter than 128 tokens."""
     target = TARGET_WORKGROUPS if target_wgs is None else target_wgs
     unit = 4 * block_size
     max_len = max(int(max_len), 1)
@@ -50,6 +52,57 @@ def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
                torch.empty(grow, dtype=torch.float32, device=device))
         _scratch[key] = cur
     return cur
+
+
+def _split_for(infer_state, model_config, engine_config):
+    n = infer_state.num_decoding_seqs
+    max_len = infer_state.num_seq_blocks * infer_state.seq_block_size
+    known = getattr(infer_state, "max_decoding_len", 0)
+    if known:
+        max_len = min(max_len, int(known)) if max_len > 0 else int(known)
+    if SPLIT_POLICY == "reference":
+        return infer_state.seq_block_size, max(1, infer_state.num_seq_blocks)
+    return choose_split(n, model_config.num_kv_heads, max_len, engine_config.block_size)
+
+
+def decode_append_and_attend(
+    k: torch.Tensor,                    # [num_tokens, num_kv_heads, head_dim]; decode rows are the tail
+    v: torch.Tensor,
+    q: torch.Tensor,                    # [num_decoding_seqs, num_q_heads, head_dim]
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_cache_new: List[torch.Tensor],
+    v_cache_new: List[torch.Tensor],
+    block_table: torch.Tensor,
+    model_config,
+    engine_config,
+    infer_state,
+    cur_layer: int,
+    o: torch.Tensor,
+) -> None:
+    """``store_kvcache`` followed by ``paged_attention`` for a decode-only batch
+    (MorphServe/worker/layers/transformer_layer.py:116-126, :181-187) as a single
+    kernel launch per layer: the new token is written to its cache slot by the
+    workgroup that attends over the sequence's last block."""
+    assert infer_state.num_prefill_seqs == 0, "the fused call covers decode-only batches"
+    assert k.is_contiguous() and v.is_contiguous() and q.is_contiguous() and o.is_contiguous()
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and block_table.is_contiguous()
+    assert infer_state.seq_block_size % engine_config.block_size == 0
+    assert q.dtype == torch.float16 and o.dtype == torch.float16 and k.dtype == torch.float16
+    n = infer_state.num_decoding_seqs
+    if n == 0:
+        return
+    hq, d = model_config.num_q_heads, model_config.head_dim
+    tps, splits = _split_for(infer_state, model_config, engine_config)
+    pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
+    mid_o, mid_lse = (None, None)
+    if splits > 1:
+        mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
+    _capi.check(_capi.lib().mkv_decode_append_attn(
+        k.data_ptr(), v.data_ptr(), q.data_ptr(), o.data_ptr(), C.byref(pool),
+        block_table.data_ptr(), block_table.shape[1], infer_state.seq_ids.data_ptr(),
+        infer_state.decoding_seq_lens.data_ptr(), n, hq, float(infer_state.softmax_scale),
+        cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
 
 
 def paged_attention(
@@ -80,14 +133,7 @@ def paged_attention(
     d = model_config.head_dim
     block_size = engine_config.block_size
 
-    max_len = infer_state.num_seq_blocks * infer_state.seq_block_size
-    known = getattr(infer_state, "max_decoding_len", 0)
-    if known:
-        max_len = min(max_len, int(known)) if max_len > 0 else int(known)
-    if SPLIT_POLICY == "reference":
-        tps, splits = infer_state.seq_block_size, max(1, infer_state.num_seq_blocks)
-    else:
-        tps, splits = choose_split(n, model_config.num_kv_heads, max_len, block_size)
+    tps, splits = _split_for(infer_state, model_config, engine_config)
 
     lib = _capi.lib()
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)

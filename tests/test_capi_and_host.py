@@ -88,6 +88,8 @@ def test_choose_split_properties():
         assert tps % 64 == 0 and tps > 0
         assert splits >= 1 and splits * tps >= max_len and (splits - 1) * tps < max_len
     assert choose_split(64, 8, 1536, 16, target_wgs=1536) == (512, 3)
+    assert choose_split(64, 8, 1536, 16) == (1536, 1)
+    assert choose_split(8, 32, 512, 16) == (256, 2)
     assert choose_split(1000, 32, 512, 16, target_wgs=1536) == (512, 1)
 
 

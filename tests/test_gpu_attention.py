@@ -10,14 +10,14 @@ import torch
 from oracle import ref_cpu as R
 from helpers import Cfg, assert_attn_close, make_case, rand_f16
 from gpu_helpers import bits, configs, to_gpu
-from morphserve_amd import build_infer_state, paged_attention, store_kvcache
+from morphserve_amd import _capi, build_infer_state, paged_attention, store_kvcache
 from morphserve_amd.worker.kernels import paged_attn as PA
 
 pytestmark = pytest.mark.gpu
 
 
 def _attend(case, dev, q, layer, policy="auto", target_wgs=None, k_new=(), v_new=(), st=None,
-            tensors=None):
+            tensors=None, variant=0):
     kc, vc, bt = tensors if tensors is not None else to_gpu(case, dev)
     model, engine = configs(case)
     if st is None:
@@ -26,6 +26,7 @@ def _attend(case, dev, q, layer, policy="auto", target_wgs=None, k_new=(), v_new
     # o arrives 2-D [n, Hq*D] in the reference's layer (a row slice of the hidden state)
     o = torch.full((n, case.Hq * case.D), float("nan"), dtype=torch.float16, device=dev)
     old = (PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS)
+    _capi.check(_capi.lib().mkv_set_decode_variant(variant))   # 0 auto, 1 vector ALU, 2 matrix cores
     PA.SPLIT_POLICY = policy
     if target_wgs is not None:
         PA.TARGET_WORKGROUPS = target_wgs
@@ -34,6 +35,7 @@ def _attend(case, dev, q, layer, policy="auto", target_wgs=None, k_new=(), v_new
                         engine, st, layer, o)
     finally:
         PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS = old
+        _capi.lib().mkv_set_decode_variant(0)
     torch.cuda.synchronize()
     return o.cpu().numpy().reshape(n, case.Hq, case.D)
 
@@ -45,14 +47,15 @@ def _oracle(case, q, layer):
 
 @pytest.mark.parametrize("Hq,Hkv", [(32, 32), (8, 4), (32, 8), (64, 8)])
 @pytest.mark.parametrize("policy", ["auto", "reference"])
-def test_decode_attention_group_sizes(cuda, Hq, Hkv, policy):
+@pytest.mark.parametrize("variant", [1, 2])
+def test_decode_attention_group_sizes(cuda, Hq, Hkv, policy, variant):
     rng = np.random.default_rng(Hq * 100 + Hkv)
     lens = [1, 2, 15, 16, 17, 63, 64, 65, 100, 333, 512, 777]
     nblk = sum((x + 15) // 16 for x in lens) + 5
     case = make_case(Hq + Hkv, 2, Hq, Hkv, lens, num_blocks=nblk, fill="all")
     q = rand_f16(rng, len(lens), Hq, case.D)
-    got = _attend(case, cuda, q, 1, policy=policy)
-    assert_attn_close(got, _oracle(case, q, 1), f"Hq={Hq} Hkv={Hkv} {policy}")
+    got = _attend(case, cuda, q, 1, policy=policy, variant=variant)
+    assert_attn_close(got, _oracle(case, q, 1), f"Hq={Hq} Hkv={Hkv} {policy} variant={variant}")
 
 
 def test_decode_attention_closed_forms(cuda):
@@ -84,8 +87,9 @@ def test_decode_attention_tail_garbage_is_masked(cuda):
         last = case.block_table[case.seq_ids[i], (n - 1) // 16]
         case.k_pool[last, 0, :, n % 16:, :] = np.float16("nan")
         case.v_pool[last, 0, :, n % 16:, :] = np.float16("inf")
-    got = _attend(case, cuda, q, 0)
-    assert_attn_close(got, want, "garbage tail")
+    for variant in (1, 2):
+        got = _attend(case, cuda, q, 0, variant=variant)
+        assert_attn_close(got, want, f"garbage tail variant={variant}")
 
 
 def test_decode_attention_split_and_permutation_invariance(cuda):
@@ -106,9 +110,10 @@ def test_decode_attention_split_and_permutation_invariance(cuda):
                          np.asarray(lens), 0)
         want = _oracle(case, q, 0)
         for wgs in (1, 64, 1536, 100000):
-            got = _attend(case, cuda, q, 0, target_wgs=wgs)
-            assert_attn_close(got, want, f"permute={permute} target_wgs={wgs}")
-            outs.append(got)
+            for variant in (1, 2):
+                got = _attend(case, cuda, q, 0, target_wgs=wgs, variant=variant)
+                assert_attn_close(got, want, f"permute={permute} target_wgs={wgs} variant={variant}")
+                outs.append(got)
     for o in outs[1:]:
         assert np.abs(o.astype(np.float64) - outs[0].astype(np.float64)).max() <= 2e-3
 
@@ -146,3 +151,40 @@ def test_decode_attention_config2_batch_one_layer(cuda):
     q = rand_f16(rng, 64, 32, 128)
     got = _attend(case, cuda, q, layer)
     assert_attn_close(got, _oracle(case, q, layer), "config 2 batch")
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 32), (32, 8), (64, 8)])
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("target_wgs", [1, 100000])
+def test_fused_append_and_attend(cuda, Hq, Hkv, variant, target_wgs):
+    """One launch per layer doing store_kvcache + paged_attention: the cache must
+    end up bit-identical to the oracle's append, the output within tolerance, for
+    last-token slots at every position of a block (first, last, middle)."""
+    from morphserve_amd import decode_append_and_attend
+    rng = np.random.default_rng(Hq + variant)
+    lens = [1, 2, 16, 17, 32, 33, 48, 100, 255, 256, 257, 1000]
+    nblk = sum((x + 15) // 16 for x in lens) + 4
+    case = make_case(Hq * 7 + Hkv, 2, Hq, Hkv, lens, num_blocks=nblk, fill="all")
+    kc, vc, bt = to_gpu(case, cuda)
+    n = len(lens)
+    q = rand_f16(rng, n, Hq, case.D)
+    k = rand_f16(rng, n, Hkv, case.D)
+    v = rand_f16(rng, n, Hkv, case.D)
+    R.append_decode(case.arena, case.lay, k, v, case.block_table, case.seq_ids, case.seq_lens, 1)
+    want = _oracle(case, q, 1)
+    model, engine = configs(case)
+    st = build_infer_state([], case.seq_ids.tolist(), case.seq_lens.tolist(), case.Hkv, case.D)
+    o = torch.full((n, Hq * case.D), float("nan"), dtype=torch.float16, device=cuda)
+    old = PA.TARGET_WORKGROUPS
+    PA.TARGET_WORKGROUPS = target_wgs
+    _capi.check(_capi.lib().mkv_set_decode_variant(variant))
+    try:
+        decode_append_and_attend(torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda),
+                                 torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, 1, o)
+    finally:
+        PA.TARGET_WORKGROUPS = old
+        _capi.lib().mkv_set_decode_variant(0)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(kc), bits(case.k_pool)), "K cache after the fused append"
+    assert np.array_equal(bits(vc), bits(case.v_pool)), "V cache after the fused append"
+    assert_attn_close(o.cpu().numpy().reshape(n, Hq, case.D), want, "fused append + attention")
