@@ -29,6 +29,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch of the decode attention kernel on this workload, from the
+# FETCH_SIZE and WRITE_SIZE counters scaled by a device copy of known size
+# (profiles/attn_decode_phase1_mfma_cfg2_pmc_traffic.md); counters cannot be
+# collected from inside this process.
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 343_659_871
 
 
 class Cfg:
@@ -42,7 +47,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
-                    choices=["cfg2_llama3_8b_decode", "cfg3_resize"])
+                    choices=["cfg2_llama3_8b_decode", "cfg3_resize", "copy_calibration"])
     ap.add_argument("--pool-blocks", type=int, default=65536)
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -166,6 +171,7 @@ def bench_decode(args):
     other_ms = (time.perf_counter() - t0) * 1e3 / reps
 
     # -- dominant kernel: per-launch duration with HIP events on its stream -------------
+    # every launch bracketed by its own event pair (the pair's own cost included) ...
     _capi.prof_reset()
     _capi.prof_enable(True)
     for _ in range(3):
@@ -176,7 +182,23 @@ def bench_decode(args):
     ap_launches, ap_ms = _capi.prof_collect(_capi.K_APPEND_DECODE)
     _capi.prof_enable(False)
     _capi.prof_reset()
-    phase1_ms = total_ms / max(launches, 1)
+    bracketed_ms = total_ms / max(launches, 1)
+    # ... and, when a step is nothing but launches of that kernel (fused call, one
+    # split), one event pair around whole steps: elapsed / launches
+    phase1_ms = bracketed_ms
+    timing = "event pair around every launch"
+    if not args.unfused and p2_launches == 0 and ap_launches == 0:
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        phase1_ms = e0.elapsed_time(e1) / (args.steps * L)
+        launches = args.steps * L
+        timing = "one event pair around back-to-back launches of this kernel only"
 
     attn_bytes, append_bytes = decode_bytes_per_layer(lens, N, HQ, HKV, D, B)
     step_bytes = (attn_bytes + append_bytes) * L
@@ -209,7 +231,9 @@ def bench_decode(args):
         "step_algorithmic_bytes": step_bytes,
         "roofline": {"bound": "hbm", "kernel": "attn_decode_phase1_mfma<4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
+                     "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH if num_blocks == 65536 else None,
+                     "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
+                     "timing": timing, "avg_launch_ms_bracketed": round(bracketed_ms, 5),
                      "algorithmic_bytes_per_launch": attn_bytes,
                      "phase2_avg_ms": round(p2_ms / max(p2_launches, 1), 5) if p2_launches else None,
                      "append_avg_ms": round(ap_ms / max(ap_launches, 1), 5) if ap_launches else None},
@@ -340,6 +364,40 @@ def bench_resize(args):
     }
 
 
+def bench_copy_calibration(args):
+    """A plain device copy of known size (the migration kernel moving 512 blocks of
+    2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
+    counters of the other kernels are scaled by."""
+    import ctypes as C
+    import torch
+    from morphserve_amd import _capi
+
+    dev = torch.device("cuda:0")
+    L, HKV, D, B = 32, 8, 128, 16
+    nb, moves = 2048, 512
+    k = torch.zeros((nb, L, HKV, B, D), dtype=torch.float16, device=dev)
+    v = torch.zeros_like(k)
+    pool = _capi.make_pool(k, v)
+    src = torch.arange(1024, 1024 + moves, dtype=torch.int64, device=dev)
+    dst = torch.arange(0, moves, dtype=torch.int64, device=dev)
+    stream = _capi.current_stream()
+    _capi.prof_reset()
+    _capi.prof_enable(True)
+    for _ in range(max(args.steps, 1)):
+        _capi.check(_capi.lib().mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream))
+    torch.cuda.synchronize()
+    launches, ms = _capi.prof_collect(_capi.K_MIGRATE)
+    _capi.prof_enable(False)
+    _capi.prof_reset()
+    moved = moves * 2 * (L * HKV * B * D * 2)
+    avg = ms / max(launches, 1)
+    return {"metric": "plain device copy GB/s (read+write)", "value": round(2 * moved / (avg * 1e-3) / 1e9, 1),
+            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 0, "ms_per_step": round(avg, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "copy_calibration: pool_migrate_kernel, 512 moves x 2 MiB (K+V)"},
+            "bytes_read_per_launch": moved, "bytes_written_per_launch": moved}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -352,7 +410,8 @@ def main():
         sys.exit(1)
     from morphserve_amd import _capi
     _capi.lib()
-    out = bench_decode(args) if args.workload == "cfg2_llama3_8b_decode" else bench_resize(args)
+    out = {"cfg2_llama3_8b_decode": bench_decode, "cfg3_resize": bench_resize,
+           "copy_calibration": bench_copy_calibration}[args.workload](args)
     print(json.dumps(out))
 
 
