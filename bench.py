@@ -47,8 +47,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
-                    choices=["cfg2_llama3_8b_decode", "cfg3_resize", "copy_calibration"])
-    ap.add_argument("--pool-blocks", type=int, default=65536)
+                    choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
+                             "copy_calibration"])
+    ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
                     help="time store_kvcache + paged_attention as two calls per layer (default: the fused "
@@ -74,11 +75,17 @@ def bench_decode(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
+    if args.workload == "cfg5_codellama34b_decode":
+        # 48 layers, GQA 64 q / 8 kv heads, batch 128, pool ~200 GB of 3 MiB blocks
+        L, HQ, HKV, D, B, N = 48, 64, 8, 128, 16, 128
+        default_blocks = 63578
+    else:
+        L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
+        default_blocks = 65536
     rng = np.random.default_rng(args.seed)
     lens = rng.integers(1024, 1537, size=N).astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
-    num_blocks = args.pool_blocks
+    num_blocks = args.pool_blocks or default_blocks
     max_blocks_per_seq = 128
     max_seqs = 256
 
@@ -218,9 +225,9 @@ def bench_decode(args):
         "vs_baseline": None,
         "dtype": "f16 (fp32 accumulate)",
         "data": "synthetic",
-        "config": {"workload": "cfg2_llama3_8b_decode: 32 layers, GQA 32q/8kv, head_dim 128, block 16, "
-                               f"batch 64, ctx U[1024,1536], pool {num_blocks} blocks "
-                               f"({num_blocks * 2 // 1024} GiB), permuted tables",
+        "config": {"workload": f"{args.workload}: {L} layers, GQA {HQ}q/{HKV}kv, head_dim 128, block 16, "
+                               f"batch {N}, ctx U[1024,1536], pool {num_blocks} blocks "
+                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), permuted tables",
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
                    "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},
@@ -229,9 +236,10 @@ def bench_decode(args):
         "eager_ms_per_step": round(eager_ms, 4),
         ("fused_eager_ms_per_step" if args.unfused else "two_call_eager_ms_per_step"): round(other_ms, 4),
         "step_algorithmic_bytes": step_bytes,
-        "roofline": {"bound": "hbm", "kernel": "attn_decode_phase1_mfma<4>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH if num_blocks == 65536 else None,
+                     "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH
+                     if (args.workload, num_blocks) == ("cfg2_llama3_8b_decode", 65536) else None,
                      "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
                      "timing": timing, "avg_launch_ms_bracketed": round(bracketed_ms, 5),
                      "algorithmic_bytes_per_launch": attn_bytes,
@@ -241,12 +249,12 @@ def bench_decode(args):
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, v_new,
-                                                  HQ, HKV, D, B, attn_bytes + append_bytes)
+                                                  HQ, HKV, D, B, attn_bytes + append_bytes, L)
     return out
 
 
 def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, v_new, HQ, HKV, D, B,
-                        bytes_per_layer):
+                        bytes_per_layer, L):
     """The oracle's torch-CPU path (append + paged attention as the reference's own
     PyTorch statement) on ONE layer of the same batch; the pool on the host holds
     only the live blocks, renumbered."""
@@ -283,8 +291,8 @@ def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, 
     per_layer = t_total / reps
     return {"value": round(bytes_per_layer / per_layer / 1e9, 3), "unit": "GB/s",
             "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of 32 layers of the same batch (64 seqs, ctx 1024-1536), {reps} repetitions, "
-                      f"{per_layer * 1e3:.1f} ms per layer; x32 layers = {per_layer * 32 * 1e3:.0f} ms per step (extrapolated)",
+            "sample": f"1 of {L} layers of the same batch ({len(lens)} seqs, ctx 1024-1536), {reps} repetitions, "
+                      f"{per_layer * 1e3:.1f} ms per layer; x{L} layers = {per_layer * L * 1e3:.0f} ms per step (extrapolated)",
             "host_cpu_count": os.cpu_count()}
 
 
@@ -410,8 +418,8 @@ def main():
         sys.exit(1)
     from morphserve_amd import _capi
     _capi.lib()
-    out = {"cfg2_llama3_8b_decode": bench_decode, "cfg3_resize": bench_resize,
-           "copy_calibration": bench_copy_calibration}[args.workload](args)
+    out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
+           "cfg3_resize": bench_resize, "copy_calibration": bench_copy_calibration}[args.workload](args)
     print(json.dumps(out))
 
 

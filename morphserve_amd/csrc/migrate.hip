@@ -51,12 +51,13 @@ __global__ __launch_bounds__(kCopyThreads) void pool_migrate_kernel(
     }
 }
 
+// One 16-byte store per thread, one 4 KiB run per workgroup, plain (cached) stores:
+// on this part that shape writes fastest (a persistent grid-stride loop or
+// non-temporal stores are 15-25 % slower).
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, int64_t units,
                                                         uint8_t* __restrict__ tail, int tail_bytes) {
-    const v4u z = {0u, 0u, 0u, 0u};
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < units; i += stride)
-        __builtin_nontemporal_store(z, (v4u*)p + i);
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < units) p[i] = make_uint4(0u, 0u, 0u, 0u);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail_bytes) tail[threadIdx.x] = 0;
 }
 
@@ -102,19 +103,24 @@ int mkv_fill_zero(void* ptr, uint64_t bytes, void* stream) {
     if (bytes == 0) return MKV_OK;
     MKV_REQUIRE(ptr != nullptr, "ptr is NULL");
     MKV_REQUIRE(((uintptr_t)ptr & 15) == 0, "ptr must be 16-byte aligned");
-    const int64_t units = (int64_t)(bytes >> 4);
-    const int tail = (int)(bytes & 15);
-    int64_t want = (units + 255) / 256;
-    const int64_t cap = (int64_t)mkv::num_cus() * 16;
-    if (want > cap) want = cap;
-    if (want < 1) want = 1;
     hipStream_t s = (hipStream_t)stream;
-    {
-        mkv::ProfScope prof(MKV_K_FILL_ZERO, s);
-        hipLaunchKernelGGL(mkv::fill_zero_kernel, dim3((unsigned)want), dim3(256), 0, s, (uint4*)ptr,
-                           units, (uint8_t*)ptr + (units << 4), tail);
+    // at most 2^30 workgroups (4 TiB) per launch
+    const uint64_t max_bytes = (uint64_t)1 << 42;
+    char* cur = (char*)ptr;
+    while (bytes > 0) {
+        const uint64_t now = bytes < max_bytes ? bytes : max_bytes;
+        const int64_t units = (int64_t)(now >> 4);
+        const int tail = (int)(now & 15);
+        const int64_t grid = units > 0 ? (units + 255) / 256 : 1;
+        {
+            mkv::ProfScope prof(MKV_K_FILL_ZERO, s);
+            hipLaunchKernelGGL(mkv::fill_zero_kernel, dim3((unsigned)grid), dim3(256), 0, s, (uint4*)cur,
+                               units, (uint8_t*)cur + (units << 4), tail);
+        }
+        MKV_HIP(hipGetLastError());
+        cur += now;
+        bytes -= now;
     }
-    MKV_HIP(hipGetLastError());
     return MKV_OK;
 }
 
