@@ -316,8 +316,22 @@ def prefill_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray,
     T, Hq, D = q.shape
     Hkv = k.shape[1]
     G = Hq // Hkv
-    ft = np.float64 if math == "np64" else np.float32
     out = np.zeros((T, Hq, D), dtype=out_dtype)
+    if math == "torch32":
+        # the same expression through torch-CPU fp32 matmuls (fast enough for 512-token prompts)
+        import torch
+        for b in range(len(seq_lens)):
+            s0, n = int(start_locs[b]), int(seq_lens[b])
+            tq = torch.from_numpy(q[s0:s0 + n]).to(torch.float32).permute(1, 0, 2)                      # [Hq,n,D]
+            tk = torch.from_numpy(k[s0:s0 + n]).to(torch.float32).permute(1, 0, 2).repeat_interleave(G, 0)
+            tv = torch.from_numpy(v[s0:s0 + n]).to(torch.float32).permute(1, 0, 2).repeat_interleave(G, 0)
+            sc = torch.bmm(tq, tk.transpose(1, 2)) * softmax_scale
+            keep = torch.tril(torch.ones(n, n, dtype=torch.bool))
+            sc = torch.where(keep, sc, torch.full_like(sc, -1e20))
+            res = torch.bmm(torch.softmax(sc, dim=2), tv).permute(1, 0, 2)
+            out[s0:s0 + n] = res.numpy().astype(out_dtype)
+        return out
+    ft = np.float64 if math == "np64" else np.float32
     for b in range(len(seq_lens)):
         s0, n = int(start_locs[b]), int(seq_lens[b])
         qq = q[s0:s0 + n].astype(ft)                  # [n, Hq, D]

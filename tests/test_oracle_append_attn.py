@@ -310,6 +310,8 @@ def test_prefill_attention_vs_dense_and_decode():
         tv = torch.from_numpy(v[sl].astype(np.float64)).permute(1, 0, 2).repeat_interleave(2, 0)
         want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, is_causal=True)
         assert np.abs(o[sl] - want.permute(1, 0, 2).numpy()).max() < 1e-12
+    o32 = R.prefill_attention(q, k, v, starts, lens, D ** -0.5, out_dtype=np.float64, math="torch32")
+    assert np.abs(o32 - o).max() < 2e-6
     # last row of each sequence == decode attention over the same tokens in a paged cache
     case = make_case(41, 1, Hq, Hkv, lens, num_blocks=12, D=D, fill="live")
     R.append_prefill(case.arena, case.lay, k, v, case.block_table, case.seq_ids, starts, lens, 0)
