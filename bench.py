@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "copy_calibration"])
+                             "cfg4_mixed", "copy_calibration"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -372,6 +372,96 @@ def bench_resize(args):
     }
 
 
+def bench_mixed(args):
+    """Config 4: Llama-2-7B MHA shapes, 32 layers; one step = eight 512-token prefill
+    chunks + 120 decode sequences (contexts lognormal(6.2, 0.6) clipped to [16, 768]):
+    per layer store_kvcache (prefill + decode rows), prefill attention, decode attention."""
+    import torch
+    from morphserve_amd import _capi, build_infer_state, paged_attention, prefill_attention, store_kvcache
+
+    dev = torch.device("cuda:0")
+    L, HQ, HKV, D, B = 32, 32, 32, 128, 16
+    rng = np.random.default_rng(args.seed)
+    p_lens = [512] * 8
+    d_lens = np.clip(rng.lognormal(6.2, 0.6, size=120), 16, 768).astype(np.int32)
+    lens = np.concatenate([np.asarray(p_lens, dtype=np.int32), d_lens])
+    nblk = (lens.astype(np.int64) + B - 1) // B
+    num_blocks = args.pool_blocks or 8192                       # 8 MiB per block (K+V): 64 GiB
+    perm = rng.permutation(num_blocks)
+    n_seq = len(lens)
+    seq_ids = rng.permutation(256)[:n_seq].astype(np.int32)
+    table = np.full((256, 64), -1, dtype=np.int32)
+    pos = 0
+    for i in range(n_seq):
+        table[seq_ids[i], :nblk[i]] = perm[pos:pos + nblk[i]]
+        pos += nblk[i]
+    shape = (num_blocks, L, HKV, B, D)
+    k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+    v_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    live_t = torch.from_numpy(perm[:pos].copy()).to(dev)
+    for c0 in range(0, pos, 64):
+        idx = live_t[c0:c0 + 64]
+        k_cache[idx] = torch.randn((len(idx), *shape[1:]), dtype=torch.float16, device=dev, generator=g)
+        v_cache[idx] = torch.randn((len(idx), *shape[1:]), dtype=torch.float16, device=dev, generator=g)
+    bt = torch.from_numpy(table).to(dev)
+    T = sum(p_lens)
+    n_tok = T + len(d_lens)
+    q = torch.randn((n_tok, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    k = torch.randn((n_tok, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    v = torch.randn((n_tok, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((n_tok, HQ * D), dtype=torch.float16, device=dev)
+    model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
+    engine = Cfg(block_size=B, max_blocks_per_seq=64)
+    st = build_infer_state(p_lens, seq_ids.tolist(), d_lens.tolist(), HKV, D)
+
+    def step():
+        for layer in range(L):
+            store_kvcache(k, v, k_cache, v_cache, [], [], bt, model, engine, st, layer)
+            prefill_attention(q[:T], k[:T], v[:T], o[:T].view(T, HQ, D), model, engine, st)
+            paged_attention(q[T:], k_cache, v_cache, [], [], bt, model, engine, st, layer, o[T:])
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    _capi.prof_reset()
+    _capi.prof_enable(True)
+    step()
+    torch.cuda.synchronize()
+    avg = {}
+    for name, kid in (("prefill_attn", _capi.K_PREFILL_ATTN), ("append_prefill", _capi.K_APPEND_PREFILL),
+                      ("append_decode", _capi.K_APPEND_DECODE), ("attn_phase1", _capi.K_ATTN_PHASE1),
+                      ("attn_phase2", _capi.K_ATTN_PHASE2)):
+        cnt, ms = _capi.prof_collect(kid)
+        avg[name] = ms / cnt if cnt else None
+    _capi.prof_enable(False)
+    _capi.prof_reset()
+    flops = sum(HQ * 4 * D * (n * n) / 2 for n in p_lens)                  # causal half, QK^T + PV
+    tflops = flops / (avg["prefill_attn"] * 1e-3) / 1e12
+    append_bytes = 2 * T * 2 * HKV * D * 2
+    dec_bytes, _ = decode_bytes_per_layer(d_lens, len(d_lens), HQ, HKV, D, B)
+    return {
+        "metric": "mixed chunked-prefill + decode step, 1 MI355X", "value": round(ms_per_step, 3), "unit": "ms/step",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": "cfg4_mixed: 32 layers, MHA 32/32, head_dim 128, 8 x 512-token prefill + 120 decode "
+                               f"(ctx lognormal(6.2,0.6) in [16,768]), pool {num_blocks} blocks"},
+        "kernel_avg_ms": {kk: (round(vv, 5) if vv is not None else None) for kk, vv in avg.items()},
+        "prefill_attn_TFLOPs": round(tflops, 1), "prefill_flops_per_layer": flops,
+        "append_prefill_GBs": round(append_bytes / (avg["append_prefill"] * 1e-3) / 1e9, 1),
+        "decode_attn_GBs": round(dec_bytes / (avg["attn_phase1"] * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false>", "achieved": round(tflops, 1),
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4), "traffic": None},
+    }
+
+
 def bench_copy_calibration(args):
     """A plain device copy of known size (the migration kernel moving 512 blocks of
     2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
@@ -419,7 +509,8 @@ def main():
     from morphserve_amd import _capi
     _capi.lib()
     out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
-           "cfg3_resize": bench_resize, "copy_calibration": bench_copy_calibration}[args.workload](args)
+           "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
+           "copy_calibration": bench_copy_calibration}[args.workload](args)
     print(json.dumps(out))
 
 
