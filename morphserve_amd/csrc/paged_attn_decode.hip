@@ -336,6 +336,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef short v4s __attribute__((ext_vector_type(4)));
 
 static constexpr int kLdsRow = 272;                 // 256 data bytes + 16 pad: conflict-free b128 rows
 static constexpr int kLdsTile = kB * kLdsRow;
@@ -402,7 +403,12 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     char* vl = stage[wave][1];
     const int wr_off = c * kLdsRow + n * 16;                     // load x of lane (c, n): token 4x + c, bytes 16n..
     const char* k_rd = kl + n * kLdsRow + c * 64;                // token row n, 64 bytes of it
-    const _Float16* v_rd = (const _Float16*)(vl + 4 * c * kLdsRow) + n;   // tokens 4c.., dim n of each tile
+    // V^T operand through the transposing LDS read (ds_read_b64_tr_b16): within a
+    // 16-lane group lane r supplies the address of four consecutive halves and
+    // lane 4a+b receives element b of the rows supplied by lanes a, a+4, a+8, a+12.
+    // Lane r therefore points at token 4c + r/4, dims 4*(r%4).. of the tile, and
+    // lane n ends up with tokens 4c..4c+3 of dim n -- the A-operand order.
+    const char* v_rd = vl + (4 * c + (n >> 2)) * kLdsRow + (n & 3) * 8;
 
     auto issue_loads = [&](int32_t pid, v4u (&kg)[4], v4u (&vg)[4]) {
         BlockAddr a = block_addr(pool, pid, block_bytes);
@@ -480,11 +486,8 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         const v4h pb = (v4h){(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3]};
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            v4h va;
-            va[0] = v_rd[0 * (kLdsRow / 2) + 16 * t];
-            va[1] = v_rd[1 * (kLdsRow / 2) + 16 * t];
-            va[2] = v_rd[2 * (kLdsRow / 2) + 16 * t];
-            va[3] = v_rd[3 * (kLdsRow / 2) + 16 * t];
+            const v4h va = __builtin_bit_cast(v4h, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (v4s __attribute__((address_space(3)))*)(v_rd + 32 * t)));
             oacc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, pb, oacc[t], 0, 0, 0);
         }
         wave_lds_fence();                            // reads done before the next tile is staged
