@@ -55,6 +55,8 @@ def parse_args():
                     help="time store_kvcache + paged_attention as two calls per layer (default: the fused "
                          "one-launch-per-layer call)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ctx", type=int, nargs=2, default=[1024, 1536], metavar=("LO", "HI"),
+                    help="decode workloads: context lengths are uniform in [LO, HI] (at most 2048)")
     ap.add_argument("--seed", type=int, default=2)
     return ap.parse_args()
 
@@ -83,7 +85,7 @@ def bench_decode(args):
         L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
         default_blocks = 65536
     rng = np.random.default_rng(args.seed)
-    lens = rng.integers(1024, 1537, size=N).astype(np.int32)
+    lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     num_blocks = args.pool_blocks or default_blocks
     max_blocks_per_seq = 128
@@ -226,7 +228,7 @@ def bench_decode(args):
         "dtype": "f16 (fp32 accumulate)",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {L} layers, GQA {HQ}q/{HKV}kv, head_dim 128, block 16, "
-                               f"batch {N}, ctx U[1024,1536], pool {num_blocks} blocks "
+                               f"batch {N}, ctx U[{args.ctx[0]},{args.ctx[1]}], pool {num_blocks} blocks "
                                f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), permuted tables",
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
@@ -291,7 +293,7 @@ def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, 
     per_layer = t_total / reps
     return {"value": round(bytes_per_layer / per_layer / 1e9, 3), "unit": "GB/s",
             "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of {L} layers of the same batch ({len(lens)} seqs, ctx 1024-1536), {reps} repetitions, "
+            "sample": f"1 of {L} layers of the same batch ({len(lens)} seqs, ctx {int(min(lens))}-{int(max(lens))}), {reps} repetitions, "
                       f"{per_layer * 1e3:.1f} ms per layer; x{L} layers = {per_layer * L * 1e3:.0f} ms per step (extrapolated)",
             "host_cpu_count": os.cpu_count()}
 

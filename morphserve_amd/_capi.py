@@ -91,11 +91,12 @@ def lib() -> C.CDLL:
     """Load the library (once).  Raises when it has not been built."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        path = os.environ.get("MORPHKV_LIBRARY") or LIB_PATH     # another build of the same ABI, for A/B runs
+        if not os.path.exists(path):
             raise ImportError(
-                f"{LIB_PATH} is missing: build it with `python -m morphserve_amd.csrc.build` "
+                f"{path} is missing: build it with `python -m morphserve_amd.csrc.build` "
                 "(there is no fallback path)")
-        handle = C.CDLL(LIB_PATH)
+        handle = C.CDLL(path)
         for name, argtypes in PROTOTYPES.items():
             fn = getattr(handle, name)
             fn.argtypes = argtypes

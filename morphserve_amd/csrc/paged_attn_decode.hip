@@ -338,8 +338,9 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef short v4s __attribute__((ext_vector_type(4)));
 
-static constexpr int kLdsRow = 272;                 // 256 data bytes + 16 pad: conflict-free b128 rows
-static constexpr int kLdsTile = kB * kLdsRow;
+static constexpr int kLdsRow = 272;                 // K rows: 256 data bytes + 16 pad: conflict-free b128 row reads
+static constexpr int kLdsRowV = 288;                // V rows 8 banks apart: conflict-free transposing reads
+static constexpr int kLdsTile = kB * kLdsRowV;      // room for either tile
 
 struct FullTag { static constexpr bool value = false; };    // a block of 16 valid tokens
 struct FinalTag { static constexpr bool value = true; };    // the sequence's last block: masked
@@ -402,13 +403,14 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     char* kl = stage[wave][0];
     char* vl = stage[wave][1];
     const int wr_off = c * kLdsRow + n * 16;                     // load x of lane (c, n): token 4x + c, bytes 16n..
+    const int wr_off_v = c * kLdsRowV + n * 16;
     const char* k_rd = kl + n * kLdsRow + c * 64;                // token row n, 64 bytes of it
     // V^T operand through the transposing LDS read (ds_read_b64_tr_b16): within a
     // 16-lane group lane r supplies the address of four consecutive halves and
     // lane 4a+b receives element b of the rows supplied by lanes a, a+4, a+8, a+12.
     // Lane r therefore points at token 4c + r/4, dims 4*(r%4).. of the tile, and
     // lane n ends up with tokens 4c..4c+3 of dim n -- the A-operand order.
-    const char* v_rd = vl + (4 * c + (n >> 2)) * kLdsRow + (n & 3) * 8;
+    const char* v_rd = vl + (4 * c + (n >> 2)) * kLdsRowV + (n & 3) * 8;
 
     auto issue_loads = [&](int32_t pid, v4u (&kg)[4], v4u (&vg)[4]) {
         BlockAddr a = block_addr(pool, pid, block_bytes);
@@ -424,7 +426,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
             *(v4u*)(kl + wr_off + x * 4 * kLdsRow) = kg[x];
-            *(v4u*)(vl + wr_off + x * 4 * kLdsRow) = vg[x];
+            *(v4u*)(vl + wr_off_v + x * 4 * kLdsRowV) = vg[x];
         }
         wave_lds_fence();
     };
@@ -450,7 +452,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
             BlockAddr a = block_addr(pool, pid, block_bytes);
             const int64_t slot = head_off + (int64_t)off * (kD * 2) + n * 16;
             *(v4u*)(const_cast<char*>(is_v ? a.v : a.k) + slot) = val;
-            *(v4u*)((is_v ? vl : kl) + off * kLdsRow + n * 16) = val;
+            *(v4u*)((is_v ? vl + off * kLdsRowV : kl + off * kLdsRow) + n * 16) = val;
         }
         wave_lds_fence();
     };

@@ -1,12 +1,17 @@
 // Causal (chunked-)prefill attention on the gfx950 matrix cores.
 //
-// One workgroup (4 waves) per (64-row query tile, q head, sequence); a wave owns
-// 16 query rows.  K/V tiles of 64 keys are staged once per workgroup in LDS.
-// Scores are produced TRANSPOSED, S^T = K Q^T (mfma 16x16x16 f16, fp32
-// accumulate), so the accumulator layout of S^T (lane = query row, registers =
-// four consecutive keys) is exactly the B-operand layout of the second product
-// O^T = V^T P^T: probabilities go from the softmax straight back into the
-// matrix core without any cross-lane movement.  Online softmax in fp32, base 2;
+// One workgroup (kWaves waves) per (16*kU*kWaves-row query tile, q head, sequence);
+// a wave owns kU 16-row column tiles.  K/V tiles of 64 keys are staged once
+// per workgroup in LDS (row-major, rows padded to 272 bytes); the global loads of
+// the next tile are in flight while the current one is consumed.
+//   S^T[key, row] = K[key, :] . Q^T        v_mfma_f32_16x16x32_f16, 4 per 16x16 tile
+//   O^T[dim, row] += V^T[dim, key] . P^T   v_mfma_f32_16x16x32_f16 over 32 keys
+// Scores are produced TRANSPOSED so that the accumulator layout of S^T (lane =
+// query row, registers = four consecutive keys) is the B-operand layout of the
+// second product: two 16-key score tiles side by side are its eight k-slots.
+// V^T comes out of the row-major V tile through the transposing LDS read
+// (ds_read_b64_tr_b16).  Every A operand (K rows, V^T) is read from LDS once
+// and used for both of the wave's column tiles.  Online softmax in fp32, base 2;
 // a query row's running max is reduced over the four lane groups that share it.
 //
 // Two K/V sources: the batch's own contiguous k, v ([T, Hkv, D]) -- the
@@ -17,13 +22,21 @@
 
 namespace mkv {
 
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef short v4s __attribute__((ext_vector_type(4)));
 
 static constexpr int kPD = 128;             // head dim
-static constexpr int kQTile = 64;           // query rows per workgroup
 static constexpr int kKTile = 64;           // keys staged per iteration
-static constexpr int kRowBytes = 272;       // LDS row stride: 256 data + 16 pad (bank spread)
+static constexpr int kU = 1;                // 16-row column tiles per wave
+static constexpr int kWaves = 8;            // waves per workgroup
+static constexpr int kThreads = 64 * kWaves;
+static constexpr int kQTile = 16 * kU * kWaves;   // query rows per workgroup
+static constexpr int kFetchSteps = (kKTile * 16) / kThreads;   // 16-byte units per thread per K (or V) tile
+static constexpr bool kPrefetch = true;     // next tile's global loads issued before the current tile's math
+static constexpr int kRowBytes = 272;       // K tile row stride: 256 data + 16 pad -> conflict-free b128 row reads
+static constexpr int kRowBytesV = 288;      // V tile row stride: rows 8 banks apart -> conflict-free transposing reads
 static constexpr float kPNegBig = -1.0e30f;
 static constexpr float kPLog2e = 1.442695040888963f;
 
@@ -42,24 +55,35 @@ struct PrefillArgs {
     int32_t num_kv_heads;
     int32_t layer;
     float scale2;
+    int32_t num_seqs;
+    int32_t num_q_tiles;          // ceil(max_len / kQTile)
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <bool PAGED>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
     __shared__ __attribute__((aligned(16))) char k_lds[kKTile * kRowBytes];
-    __shared__ __attribute__((aligned(16))) char v_lds[kKTile * kRowBytes];
+    __shared__ __attribute__((aligned(16))) char v_lds[kKTile * kRowBytesV];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int m = lane & 15;          // query row (B / C column) or key / dim row (A)
+    const int m = lane & 15;          // query row of a column tile (B / C), key or dim row (A)
     const int c = lane >> 4;          // lane group
-    const int qt = blockIdx.x;
-    const int hq = blockIdx.y;
-    const int b = blockIdx.z;
+    // Workgroup id -> (query tile, q head, sequence).  Consecutive ids go to the
+    // eight XCDs in turn and every XCD has its own L2, so the id's low three bits
+    // pick the (sequence, head) pair's residue and ALL query tiles of a pair land
+    // on one XCD: the pair's K/V is fetched into that L2 once and shared by its
+    // tiles.  Longest tiles (most keys) first.
     const int Hq = a.num_q_heads;
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    const int qt = a.num_q_tiles - 1 - slot % a.num_q_tiles;
+    const int pair = (slot / a.num_q_tiles) * 8 + xcd;
+    if (pair >= Hq * a.num_seqs) return;
+    const int hq = pair % Hq;
+    const int b = pair / Hq;
     const int Hkv = a.num_kv_heads;
     const int kvh = hq / (Hq / Hkv);
 
@@ -68,53 +92,61 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillArgs a, 
     if (q0 >= len) return;
     const int64_t start = a.start_locs[b];
     const int prefix = (PAGED && a.prefix_lens) ? a.prefix_lens[b] : 0;
-    const int kv_len = prefix + min(len, q0 + kQTile);       // keys this tile can see
-    const int my_row = q0 + wave * 16 + m;                   // chunk-local query row of this lane
-    const int my_pos = prefix + my_row;                      // its position in the sequence
-    const int wave_max_pos = prefix + min(len - 1, q0 + wave * 16 + 15);
+    const int kv_len = prefix + min(len, q0 + kQTile);       // keys this workgroup can see
 
-    // Q^T as B operand: lane (row m, group c) holds dims c*32 + kk*4 .. +3, kk = 0..7
-    // (the contraction order over dims is free; K uses the same permutation).
-    v4h qb[8];
-    {
-        uint4 raw[4];
-        if (my_row < len) {
-            const uint4* qp = (const uint4*)(a.q + ((start + my_row) * Hq + hq) * kPD + c * 32);
+    // this wave's two column tiles: chunk-local rows row0[u] .. row0[u]+15
+    int my_row[kU], my_pos[kU], tile_min_pos[kU], tile_max_pos[kU];
 #pragma unroll
-            for (int x = 0; x < 4; ++x) raw[x] = qp[x];
+    for (int u = 0; u < kU; ++u) {
+        const int r0 = q0 + wave * (16 * kU) + u * 16;
+        my_row[u] = r0 + m;
+        my_pos[u] = prefix + my_row[u];
+        tile_min_pos[u] = prefix + r0;
+        tile_max_pos[u] = prefix + min(len - 1, r0 + 15);     // < tile_min_pos when the tile has no row
+    }
+
+    // Q^T as B operand: lane (row m, group c) holds dims c*32 + 8x .. +8 for product x
+    // (the contraction order over dims is free; K uses the same order).
+    v8h qb[kU][4];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        if (my_row[u] < len) {
+            const uint4* qp = (const uint4*)(a.q + ((start + my_row[u]) * Hq + hq) * kPD + c * 32);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) qb[u][x] = __builtin_bit_cast(v8h, qp[x]);
         } else {
 #pragma unroll
-            for (int x = 0; x < 4; ++x) raw[x] = make_uint4(0u, 0u, 0u, 0u);
-        }
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            const uint2 lo = make_uint2(raw[x].x, raw[x].y);
-            const uint2 hi = make_uint2(raw[x].z, raw[x].w);
-            qb[2 * x] = __builtin_bit_cast(v4h, lo);
-            qb[2 * x + 1] = __builtin_bit_cast(v4h, hi);
+            for (int x = 0; x < 4; ++x) qb[u][x] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
 
-    v4f acc[8];                       // O^T tiles: dims 16t + 4c + j, query row m
+    v4f acc[kU][8];                    // O^T tiles: dims 16t + 4c + j, query row m of column tile u
 #pragma unroll
-    for (int t = 0; t < 8; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    float m_run = kPNegBig;
-    float l_run = 0.f;                // per-lane partial of the row sum (reduced over c at the end)
+    for (int u = 0; u < kU; ++u)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[u][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+    float m_run[kU], l_run[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        m_run[u] = kPNegBig;
+        l_run[u] = 0.f;
+    }      // per-lane share of the row sums (reduced over c at the end)
 
     const int64_t block_bytes = PAGED ? pool_block_bytes(pool) : 0;
     const int64_t total_blocks = PAGED ? pool_total_blocks(pool) : 0;
     const int32_t* bt_row = PAGED ? a.block_table + (int64_t)a.seq_ids[b] * a.max_blocks_per_seq : nullptr;
 
-    for (int key0 = 0; key0 < kv_len; key0 += kKTile) {
-        __syncthreads();              // previous tile fully consumed
-        // ---- stage 64 keys of K and V in LDS (16 bytes per thread per step) ----
+    // global -> registers for one 64-key tile: 16 bytes per thread per step
+    uint4 kreg[kFetchSteps], vreg[kFetchSteps];
+    auto fetch_tile = [&](int key0) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int idx = tid + 256 * u;
+        for (int u = 0; u < kFetchSteps; ++u) {
+            const int idx = tid + kThreads * u;
             const int key = idx >> 4;
             const int ch = idx & 15;
             const int pos = key0 + key;
-            uint4 kk4 = make_uint4(0u, 0u, 0u, 0u), vv4 = kk4;
+            kreg[u] = make_uint4(0u, 0u, 0u, 0u);
+            vreg[u] = kreg[u];
             if (pos < kv_len) {
                 if (PAGED) {
                     const int64_t pid = bt_row[pos / pool.block_size];
@@ -122,106 +154,159 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillArgs a, 
                         BlockAddr ba = block_addr(pool, pid, block_bytes);
                         const int64_t off = ((int64_t)a.layer * Hkv + kvh) * ((int64_t)pool.block_size * kPD * 2) +
                                             (int64_t)(pos % pool.block_size) * (kPD * 2) + ch * 16;
-                        kk4 = *(const uint4*)(ba.k + off);
-                        vv4 = *(const uint4*)(ba.v + off);
+                        kreg[u] = *(const uint4*)(ba.k + off);
+                        vreg[u] = *(const uint4*)(ba.v + off);
                     }
                 } else {
                     const int64_t off = ((start + pos) * Hkv + kvh) * kPD + ch * 8;
-                    kk4 = *(const uint4*)(a.k + off);
-                    vv4 = *(const uint4*)(a.v + off);
+                    kreg[u] = *(const uint4*)(a.k + off);
+                    vreg[u] = *(const uint4*)(a.v + off);
                 }
             }
-            *(uint4*)(k_lds + key * kRowBytes + ch * 16) = kk4;
-            *(uint4*)(v_lds + key * kRowBytes + ch * 16) = vv4;
+        }
+    };
+
+    const char* k_rd = k_lds + m * kRowBytes + c * 64;                       // + 16n rows, + 16x bytes
+    const char* v_rd = v_lds + (4 * c + (m >> 2)) * kRowBytesV + (m & 3) * 8;  // + 16n rows, + 32t bytes
+
+    if (kPrefetch) fetch_tile(0);
+    for (int key0 = 0; key0 < kv_len; key0 += kKTile) {
+        if (!kPrefetch) fetch_tile(key0);
+        __syncthreads();              // previous tile fully consumed
+#pragma unroll
+        for (int u = 0; u < kFetchSteps; ++u) {
+            const int idx = tid + kThreads * u;
+            *(uint4*)(k_lds + (idx >> 4) * kRowBytes + (idx & 15) * 16) = kreg[u];
+            *(uint4*)(v_lds + (idx >> 4) * kRowBytesV + (idx & 15) * 16) = vreg[u];
         }
         __syncthreads();
+        if (kPrefetch && key0 + kKTile < kv_len) fetch_tile(key0 + kKTile);   // in flight during the math below
 
-        // ---- four 16-key sub-tiles ------------------------------------------------
-        float s[4][4];
-        bool live[4];
+        // ---- scores of the four 16-key sub-tiles, both column tiles ----------------------
+        float s[kU][4][4];
+        bool live[kU][4];
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
-            live[n] = (key0 + 16 * n) <= wave_max_pos && (key0 + 16 * n) < kv_len;   // wave-uniform
-            v4f st = (v4f){0.f, 0.f, 0.f, 0.f};
-            if (live[n]) {
-                const uint4* kr = (const uint4*)(k_lds + (16 * n + m) * kRowBytes + c * 64);
+            const int kp0 = key0 + 16 * n;
+            bool any = false;
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                live[u][n] = kp0 <= tile_max_pos[u] && kp0 < kv_len;          // wave-uniform
+                any = any || live[u][n];
+            }
+            v4f st[kU];
+#pragma unroll
+            for (int u = 0; u < kU; ++u) st[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+            if (any) {
+                const uint4* kr = (const uint4*)(k_rd + 16 * n * kRowBytes);
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
-                    const uint4 w = kr[x];
-                    const v4h a0 = __builtin_bit_cast(v4h, make_uint2(w.x, w.y));
-                    const v4h a1 = __builtin_bit_cast(v4h, make_uint2(w.z, w.w));
-                    st = __builtin_amdgcn_mfma_f32_16x16x16f16(a0, qb[2 * x], st, 0, 0, 0);
-                    st = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, qb[2 * x + 1], st, 0, 0, 0);
+                    const v8h ka = __builtin_bit_cast(v8h, kr[x]);
+#pragma unroll
+                    for (int u = 0; u < kU; ++u)
+                        if (live[u][n]) st[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[u][x], st[u], 0, 0, 0);
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int key_pos = key0 + 16 * n + 4 * c + j;
-                const bool ok = live[n] && key_pos <= my_pos && key_pos < kv_len;
-                s[n][j] = ok ? st[j] * a.scale2 : kPNegBig;
+            for (int u = 0; u < kU; ++u) {
+                const bool whole = kp0 + 15 <= tile_min_pos[u] && kp0 + 15 < kv_len;   // no masking needed
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int key_pos = kp0 + 4 * c + j;
+                    const bool ok = live[u][n] && (whole || (key_pos <= my_pos[u] && key_pos < kv_len));
+                    s[u][n][j] = ok ? st[u][j] * a.scale2 : kPNegBig;
+                }
             }
         }
-        float mx = m_run;
+        // ---- online softmax per column tile -----------------------------------------------
+        v8h pb[kU][2];                 // P^T as B operand: [pair of sub-tiles] = 8 k-slots
 #pragma unroll
-        for (int n = 0; n < 4; ++n)
+        for (int u = 0; u < kU; ++u) {
+            float mx = m_run[u];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[n][j]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float alpha = pf_exp2(m_run - mx);
-        m_run = mx;
-        l_run *= alpha;
+            for (int n = 0; n < 4; ++n)
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[t] *= alpha;
-
+                for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][n][j]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            if (__ballot(mx > m_run[u]) != 0) {       // some row's max moved: rescale (wave-uniform branch)
+                const float alpha = pf_exp2(m_run[u] - mx);
+                l_run[u] *= alpha;
 #pragma unroll
-        for (int n = 0; n < 4; ++n) {
-            if (!live[n]) continue;
-            float p[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                p[j] = (s[n][j] > 0.5f * kPNegBig) ? pf_exp2(s[n][j] - mx) : 0.f;
-                l_run += p[j];
+                for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
             }
-            const v4h pb = (v4h){(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3]};
-            // A operand = V^T: lane (dim row m of tile t, group c) holds keys 4c .. 4c+3
-            const _Float16* vbase = (const _Float16*)(v_lds + (16 * n + 4 * c) * kRowBytes) + m;
+            m_run[u] = mx;
+            float p[4][4];
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    p[n][j] = (s[u][n][j] > 0.5f * kPNegBig) ? pf_exp2(s[u][n][j] - mx) : 0.f;
+                    l_run[u] += p[n][j];
+                }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                pb[u][h] = (v8h){(_Float16)p[2 * h][0],     (_Float16)p[2 * h][1],     (_Float16)p[2 * h][2],
+                                 (_Float16)p[2 * h][3],     (_Float16)p[2 * h + 1][0], (_Float16)p[2 * h + 1][1],
+                                 (_Float16)p[2 * h + 1][2], (_Float16)p[2 * h + 1][3]};
+        }
+        // ---- O^T += V^T . P^T, 32 keys per product ----------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            bool need[kU];
+            bool any_need = false;
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                need[u] = live[u][2 * h] || live[u][2 * h + 1];
+                any_need = any_need || need[u];
+            }
+            if (!any_need) continue;
+            const char* vp = v_rd + 32 * h * kRowBytesV;
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                v4h va;
-                va[0] = vbase[0 * (kRowBytes / 2) + 16 * t];
-                va[1] = vbase[1 * (kRowBytes / 2) + 16 * t];
-                va[2] = vbase[2 * (kRowBytes / 2) + 16 * t];
-                va[3] = vbase[3 * (kRowBytes / 2) + 16 * t];
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, pb, acc[t], 0, 0, 0);
+                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3)))*)(vp + 32 * t));
+                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3)))*)(vp + 16 * kRowBytesV + 32 * t));
+                const v8h va = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int u = 0; u < kU; ++u)
+                    if (need[u]) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][h], acc[u][t], 0, 0, 0);
             }
         }
     }
 
-    float l_tot = l_run + __shfl_xor(l_run, 16);
-    l_tot += __shfl_xor(l_tot, 32);
-    if (my_row < len) {
-        const float inv = 1.f / l_tot;
-        __half* op = a.o + ((start + my_row) * Hq + hq) * kPD;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const v4h out = (v4h){(_Float16)(acc[t][0] * inv), (_Float16)(acc[t][1] * inv),
-                                  (_Float16)(acc[t][2] * inv), (_Float16)(acc[t][3] * inv)};
-            *(uint2*)(op + 16 * t + 4 * c) = __builtin_bit_cast(uint2, out);
+    for (int u = 0; u < kU; ++u) {
+        float l_tot = l_run[u] + __shfl_xor(l_run[u], 16);
+        l_tot += __shfl_xor(l_tot, 32);
+        if (my_row[u] < len) {
+            const float inv = 1.f / l_tot;
+            __half* op = a.o + ((start + my_row[u]) * Hq + hq) * kPD;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const v4h out = (v4h){(_Float16)(acc[u][t][0] * inv), (_Float16)(acc[u][t][1] * inv),
+                                      (_Float16)(acc[u][t][2] * inv), (_Float16)(acc[u][t][3] * inv)};
+                *(uint2*)(op + 16 * t + 4 * c) = __builtin_bit_cast(uint2, out);
+            }
         }
     }
 }
 
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
                           int max_len, hipStream_t s) {
-    dim3 grid((unsigned)cdiv(max_len, kQTile), (unsigned)a.num_q_heads, (unsigned)num_seqs);
+    PrefillArgs args = a;
+    args.num_seqs = num_seqs;
+    args.num_q_tiles = cdiv(max_len, kQTile);
+    const int64_t pairs8 = ((int64_t)a.num_q_heads * num_seqs + 7) / 8 * 8;     // pairs padded to the XCD count
+    dim3 grid((unsigned)(pairs8 * args.num_q_tiles));
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
         if (paged) {
-            hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, dim3(256), 0, s, a, *pool);
+            hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, dim3(kThreads), 0, s, args, *pool);
         } else {
-            hipLaunchKernelGGL(prefill_attn_kernel<false>, grid, dim3(256), 0, s, a, empty);
+            hipLaunchKernelGGL(prefill_attn_kernel<false>, grid, dim3(kThreads), 0, s, args, empty);
         }
     }
     MKV_HIP(hipGetLastError());
