@@ -1,9 +1,10 @@
 // Causal (chunked-)prefill attention on the gfx950 matrix cores.
 //
-// One workgroup (kWaves waves) per (16*kU*kWaves-row query tile, q head, sequence);
-// a wave owns kU 16-row column tiles.  K/V tiles of 64 keys are staged once
-// per workgroup in LDS (row-major, rows padded to 272 bytes); the global loads of
-// the next tile are in flight while the current one is consumed.
+// One workgroup of four waves per (128-row query tile, q head, sequence); a wave
+// owns two 16-row column tiles (32 query rows).  K/V tiles of 64 keys are staged
+// per workgroup in LDS, row-major, double buffered: while one buffer is consumed
+// the next tile's global loads are in flight in registers and are written to the
+// other buffer at the end of the iteration -- one barrier per tile.
 //   S^T[key, row] = K[key, :] . Q^T        v_mfma_f32_16x16x32_f16, 4 per 16x16 tile
 //   O^T[dim, row] += V^T[dim, key] . P^T   v_mfma_f32_16x16x32_f16 over 32 keys
 // Scores are produced TRANSPOSED so that the accumulator layout of S^T (lane =
@@ -11,13 +12,18 @@
 // second product: two 16-key score tiles side by side are its eight k-slots.
 // V^T comes out of the row-major V tile through the transposing LDS read
 // (ds_read_b64_tr_b16).  Every A operand (K rows, V^T) is read from LDS once
-// and used for both of the wave's column tiles.  Online softmax in fp32, base 2;
-// a query row's running max is reduced over the four lane groups that share it.
+// and used for both of the wave's column tiles.  Online softmax in fp32, base 2,
+// on the raw scores (the scale is folded into the exponent's fma); a query row's
+// running max is reduced over the four lane groups that share it with the
+// lane-swap instructions.  Tiles entirely below a wave's diagonal take a body
+// without any masking; only the one or two diagonal tiles pay for the compares.
 //
 // Two K/V sources: the batch's own contiguous k, v ([T, Hkv, D]) -- the
 // reference's whole-prompt prefill -- or the paged cache through the block
 // table, where a chunk of queries at positions prefix .. prefix+len-1 attends to
 // everything cached up to its own position.
+#include <type_traits>
+
 #include "common.h"
 
 namespace mkv {
@@ -26,17 +32,19 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef short v4s __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 static constexpr int kPD = 128;             // head dim
 static constexpr int kKTile = 64;           // keys staged per iteration
-static constexpr int kU = 1;                // 16-row column tiles per wave
-static constexpr int kWaves = 8;            // waves per workgroup
+static constexpr int kU = 2;                // 16-row column tiles per wave
+static constexpr int kWaves = 4;            // waves per workgroup
 static constexpr int kThreads = 64 * kWaves;
 static constexpr int kQTile = 16 * kU * kWaves;   // query rows per workgroup
 static constexpr int kFetchSteps = (kKTile * 16) / kThreads;   // 16-byte units per thread per K (or V) tile
-static constexpr bool kPrefetch = true;     // next tile's global loads issued before the current tile's math
 static constexpr int kRowBytes = 272;       // K tile row stride: 256 data + 16 pad -> conflict-free b128 row reads
 static constexpr int kRowBytesV = 288;      // V tile row stride: rows 8 banks apart -> conflict-free transposing reads
+static constexpr int kKBuf = kKTile * kRowBytes;
+static constexpr int kVBuf = kKTile * kRowBytesV;
 static constexpr float kPNegBig = -1.0e30f;
 static constexpr float kPLog2e = 1.442695040888963f;
 
@@ -54,17 +62,33 @@ struct PrefillArgs {
     int32_t num_q_heads;
     int32_t num_kv_heads;
     int32_t layer;
-    float scale2;
+    float scale2;                 // softmax scale * log2(e), > 0
     int32_t num_seqs;
     int32_t num_q_tiles;          // ceil(max_len / kQTile)
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// three-input max in one instruction (the two-input form first canonicalises both operands)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// max over the four lanes {l, l^16, l^32, l^48}: swap 16-lane rows, then 32-lane halves
+__device__ __forceinline__ float max_over_groups(float x) {
+    const unsigned xi = __builtin_bit_cast(unsigned, x);
+    auto a = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);
+    x = fmaxf(__builtin_bit_cast(float, (unsigned)a[0]), __builtin_bit_cast(float, (unsigned)a[1]));
+    const unsigned yi = __builtin_bit_cast(unsigned, x);
+    auto b = __builtin_amdgcn_permlane32_swap(yi, yi, false, false);
+    return fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
+}
 template <bool PAGED>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
-    __shared__ __attribute__((aligned(16))) char k_lds[kKTile * kRowBytes];
-    __shared__ __attribute__((aligned(16))) char v_lds[kKTile * kRowBytesV];
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
+    __shared__ __attribute__((aligned(16))) char k_lds[2 * kKBuf];
+    __shared__ __attribute__((aligned(16))) char v_lds[2 * kVBuf];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -75,12 +99,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     // eight XCDs in turn and every XCD has its own L2, so the id's low three bits
     // pick the (sequence, head) pair's residue and ALL query tiles of a pair land
     // on one XCD: the pair's K/V is fetched into that L2 once and shared by its
-    // tiles.  Longest tiles (most keys) first.
+    // tiles.  A workgroup takes TWO query tiles of its sequence, the i-th from the
+    // end and the i-th from the start: under the causal mask their key counts add
+    // up to the same total for every i, so all workgroups of a sequence carry equal
+    // work.
     const int Hq = a.num_q_heads;
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    const int qt = a.num_q_tiles - 1 - slot % a.num_q_tiles;
-    const int pair = (slot / a.num_q_tiles) * 8 + xcd;
+    const int half_tiles = (a.num_q_tiles + 1) >> 1;
+    const int ti = slot % half_tiles;
+    const int pair = (slot / half_tiles) * 8 + xcd;
     if (pair >= Hq * a.num_seqs) return;
     const int hq = pair % Hq;
     const int b = pair / Hq;
@@ -88,21 +116,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     const int kvh = hq / (Hq / Hkv);
 
     const int len = a.seq_lens[b];
-    const int q0 = qt * kQTile;
-    if (q0 >= len) return;
+    const int n_qt = (len + kQTile - 1) / kQTile;            // query tiles of THIS sequence
+    if (2 * ti >= n_qt) return;
     const int64_t start = a.start_locs[b];
     const int prefix = (PAGED && a.prefix_lens) ? a.prefix_lens[b] : 0;
+
+  for (int part = 0; part < 2; ++part) {
+    const int qt = part == 0 ? n_qt - 1 - ti : ti;
+    if (part == 1 && 2 * ti == n_qt - 1) break;              // odd count: the middle tile was part 0
+    const int q0 = qt * kQTile;
     const int kv_len = prefix + min(len, q0 + kQTile);       // keys this workgroup can see
 
-    // this wave's two column tiles: chunk-local rows row0[u] .. row0[u]+15
-    int my_row[kU], my_pos[kU], tile_min_pos[kU], tile_max_pos[kU];
+    // this wave's 32 rows: chunk-local rows r0w .. r0w+31, column tile u = rows r0w+16u ..
+    const int r0w = q0 + wave * (16 * kU);
+    const int wave_min_pos = prefix + r0w;
+    const int wave_max_pos = prefix + min(len - 1, r0w + 16 * kU - 1);   // < wave_min_pos: no row at all
+    int my_row[kU], my_pos[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-        const int r0 = q0 + wave * (16 * kU) + u * 16;
-        my_row[u] = r0 + m;
+        my_row[u] = r0w + u * 16 + m;
         my_pos[u] = prefix + my_row[u];
-        tile_min_pos[u] = prefix + r0;
-        tile_max_pos[u] = prefix + min(len - 1, r0 + 15);     // < tile_min_pos when the tile has no row
     }
 
     // Q^T as B operand: lane (row m, group c) holds dims c*32 + 8x .. +8 for product x
@@ -125,97 +158,100 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     for (int u = 0; u < kU; ++u)
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[u][t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    float m_run[kU], l_run[kU];
+    // Row sums come out of the matrix cores as well: a V^T row of ones turns the second
+    // product into sum_k P^T[k, row], so every register of lsum[u] holds the row's sum of the
+    // fp16-rounded probabilities -- the same values the numerator is built from.
+    float m_run[kU];                   // running max of the RAW scores
+    v4f lsum[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
         m_run[u] = kPNegBig;
-        l_run[u] = 0.f;
-    }      // per-lane share of the row sums (reduced over c at the end)
+        lsum[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
+    const v8h ones = (v8h){1, 1, 1, 1, 1, 1, 1, 1};
 
     const int64_t block_bytes = PAGED ? pool_block_bytes(pool) : 0;
     const int64_t total_blocks = PAGED ? pool_total_blocks(pool) : 0;
     const int32_t* bt_row = PAGED ? a.block_table + (int64_t)a.seq_ids[b] * a.max_blocks_per_seq : nullptr;
 
-    // global -> registers for one 64-key tile: 16 bytes per thread per step
-    uint4 kreg[kFetchSteps], vreg[kFetchSteps];
+    // global -> registers for one 64-key tile: 16 bytes per thread per step.  Keys at or past
+    // kv_len re-read the last visible key (finite values; their scores are masked and their
+    // probabilities are zero); unmapped table entries read as zeros.
+    v4u kreg[kFetchSteps], vreg[kFetchSteps];
     auto fetch_tile = [&](int key0) {
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
             const int idx = tid + kThreads * u;
-            const int key = idx >> 4;
             const int ch = idx & 15;
-            const int pos = key0 + key;
-            kreg[u] = make_uint4(0u, 0u, 0u, 0u);
-            vreg[u] = kreg[u];
-            if (pos < kv_len) {
-                if (PAGED) {
-                    const int64_t pid = bt_row[pos / pool.block_size];
-                    if (pid >= 0 && pid < total_blocks) {
-                        BlockAddr ba = block_addr(pool, pid, block_bytes);
-                        const int64_t off = ((int64_t)a.layer * Hkv + kvh) * ((int64_t)pool.block_size * kPD * 2) +
-                                            (int64_t)(pos % pool.block_size) * (kPD * 2) + ch * 16;
-                        kreg[u] = *(const uint4*)(ba.k + off);
-                        vreg[u] = *(const uint4*)(ba.v + off);
-                    }
-                } else {
-                    const int64_t off = ((start + pos) * Hkv + kvh) * kPD + ch * 8;
-                    kreg[u] = *(const uint4*)(a.k + off);
-                    vreg[u] = *(const uint4*)(a.v + off);
+            const int pos = min(key0 + (idx >> 4), kv_len - 1);
+            if (PAGED) {
+                const int64_t pid = bt_row[pos / pool.block_size];
+                kreg[u] = (v4u){0u, 0u, 0u, 0u};
+                vreg[u] = kreg[u];
+                if (pid >= 0 && pid < total_blocks) {
+                    BlockAddr ba = block_addr(pool, pid, block_bytes);
+                    const int64_t off = ((int64_t)a.layer * Hkv + kvh) * ((int64_t)pool.block_size * kPD * 2) +
+                                        (int64_t)(pos % pool.block_size) * (kPD * 2) + ch * 16;
+                    kreg[u] = *(const v4u*)(ba.k + off);
+                    vreg[u] = *(const v4u*)(ba.v + off);
                 }
+            } else {
+                const int64_t off = ((start + pos) * Hkv + kvh) * kPD + ch * 8;
+                kreg[u] = *(const v4u*)(a.k + off);
+                vreg[u] = *(const v4u*)(a.v + off);
             }
         }
     };
-
-    const char* k_rd = k_lds + m * kRowBytes + c * 64;                       // + 16n rows, + 16x bytes
-    const char* v_rd = v_lds + (4 * c + (m >> 2)) * kRowBytesV + (m & 3) * 8;  // + 16n rows, + 32t bytes
-
-    if (kPrefetch) fetch_tile(0);
-    for (int key0 = 0; key0 < kv_len; key0 += kKTile) {
-        if (!kPrefetch) fetch_tile(key0);
-        __syncthreads();              // previous tile fully consumed
+    auto stage_tile = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
             const int idx = tid + kThreads * u;
-            *(uint4*)(k_lds + (idx >> 4) * kRowBytes + (idx & 15) * 16) = kreg[u];
-            *(uint4*)(v_lds + (idx >> 4) * kRowBytesV + (idx & 15) * 16) = vreg[u];
+            *(v4u*)(k_lds + buf * kKBuf + (idx >> 4) * kRowBytes + (idx & 15) * 16) = kreg[u];
+            *(v4u*)(v_lds + buf * kVBuf + (idx >> 4) * kRowBytesV + (idx & 15) * 16) = vreg[u];
         }
-        __syncthreads();
-        if (kPrefetch && key0 + kKTile < kv_len) fetch_tile(key0 + kKTile);   // in flight during the math below
+    };
 
-        // ---- scores of the four 16-key sub-tiles, both column tiles ----------------------
-        float s[kU][4][4];
-        bool live[kU][4];
+    const int k_rd_off = m * kRowBytes + c * 64;                            // + 16n rows, + 16x bytes
+    const int v_rd_off = (4 * c + (m >> 2)) * kRowBytesV + (m & 3) * 8;     // + 16n rows, + 32t bytes
+
+    // one 64-key tile against this wave's 32 rows
+    auto tile_body = [&](auto masked_tag, int buf, int key0) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const char* k_rd = k_lds + buf * kKBuf + k_rd_off;
+        const char* v_rd = v_lds + buf * kVBuf + v_rd_off;
+        // ---- raw scores of the four 16-key sub-tiles, both column tiles ------------------
+        // K fragments of sub-tile n+1 are requested before the products of sub-tile n, so
+        // the LDS latency is covered by eight matrix instructions
+        v4f st[kU][4];
+        uint4 kf[2][4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) kf[0][x] = ((const uint4*)k_rd)[x];
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
-            const int kp0 = key0 + 16 * n;
-            bool any = false;
+            if (n < 3) {
+                const uint4* kr = (const uint4*)(k_rd + 16 * (n + 1) * kRowBytes);
 #pragma unroll
-            for (int u = 0; u < kU; ++u) {
-                live[u][n] = kp0 <= tile_max_pos[u] && kp0 < kv_len;          // wave-uniform
-                any = any || live[u][n];
+                for (int x = 0; x < 4; ++x) kf[(n + 1) & 1][x] = kr[x];
             }
-            v4f st[kU];
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int u = 0; u < kU; ++u) st[u] = (v4f){0.f, 0.f, 0.f, 0.f};
-            if (any) {
-                const uint4* kr = (const uint4*)(k_rd + 16 * n * kRowBytes);
+            for (int u = 0; u < kU; ++u) st[u][n] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const v8h ka = __builtin_bit_cast(v8h, kr[x]);
+            for (int x = 0; x < 4; ++x) {
+                const v8h ka = __builtin_bit_cast(v8h, kf[n & 1][x]);
 #pragma unroll
-                    for (int u = 0; u < kU; ++u)
-                        if (live[u][n]) st[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[u][x], st[u], 0, 0, 0);
-                }
+                for (int u = 0; u < kU; ++u)
+                    st[u][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[u][x], st[u][n], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (MASKED) {
 #pragma unroll
-            for (int u = 0; u < kU; ++u) {
-                const bool whole = kp0 + 15 <= tile_min_pos[u] && kp0 + 15 < kv_len;   // no masking needed
+                for (int u = 0; u < kU; ++u)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int key_pos = kp0 + 4 * c + j;
-                    const bool ok = live[u][n] && (whole || (key_pos <= my_pos[u] && key_pos < kv_len));
-                    s[u][n][j] = ok ? st[u][j] * a.scale2 : kPNegBig;
-                }
+                    for (int j = 0; j < 4; ++j) {
+                        const int key_pos = key0 + 16 * n + 4 * c + j;
+                        if (!(key_pos <= my_pos[u] && key_pos < kv_len)) st[u][n][j] = kPNegBig;
+                    }
             }
         }
         // ---- online softmax per column tile -----------------------------------------------
@@ -224,26 +260,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
         for (int u = 0; u < kU; ++u) {
             float mx = m_run[u];
 #pragma unroll
-            for (int n = 0; n < 4; ++n)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[u][n][j]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            for (int n = 0; n < 4; ++n) mx = max3(max3(mx, st[u][n][0], st[u][n][1]), st[u][n][2], st[u][n][3]);
+            mx = max_over_groups(mx);
             if (__ballot(mx > m_run[u]) != 0) {       // some row's max moved: rescale (wave-uniform branch)
-                const float alpha = pf_exp2(m_run[u] - mx);
-                l_run[u] *= alpha;
+                const float alpha = pf_exp2((m_run[u] - mx) * a.scale2);
+                lsum[u] *= alpha;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
             }
             m_run[u] = mx;
+            const float ms = -mx * a.scale2;
             float p[4][4];
 #pragma unroll
             for (int n = 0; n < 4; ++n)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    p[n][j] = (s[u][n][j] > 0.5f * kPNegBig) ? pf_exp2(s[u][n][j] - mx) : 0.f;
-                    l_run[u] += p[n][j];
-                }
+                for (int j = 0; j < 4; ++j)
+                    p[n][j] = pf_exp2(__builtin_fmaf(st[u][n][j], a.scale2, ms));   // masked: exp2(-huge) = 0
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 pb[u][h] = (v8h){(_Float16)p[2 * h][0],     (_Float16)p[2 * h][1],     (_Float16)p[2 * h][2],
@@ -253,15 +285,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
         // ---- O^T += V^T . P^T, 32 keys per product ----------------------------------------
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            bool need[kU];
-            bool any_need = false;
-#pragma unroll
-            for (int u = 0; u < kU; ++u) {
-                need[u] = live[u][2 * h] || live[u][2 * h + 1];
-                any_need = any_need || need[u];
-            }
-            if (!any_need) continue;
             const char* vp = v_rd + 32 * h * kRowBytesV;
+#pragma unroll
+            for (int u = 0; u < kU; ++u)
+                lsum[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[u][h], lsum[u], 0, 0, 0);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -271,15 +298,40 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
                 const v8h va = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
                 for (int u = 0; u < kU; ++u)
-                    if (need[u]) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][h], acc[u][t], 0, 0, 0);
+                    acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][h], acc[u][t], 0, 0, 0);
             }
         }
+    };
+
+    const int num_tiles = (kv_len + kKTile - 1) / kKTile;
+    const bool wave_has_rows = r0w < len;
+    fetch_tile(0);
+    stage_tile(0);
+    __syncthreads();
+    for (int it = 0; it + 1 < num_tiles; ++it) {
+        const int buf = it & 1;
+        const int key0 = it * kKTile;
+        fetch_tile(key0 + kKTile);                    // in flight during the math below
+        if (wave_has_rows && key0 <= wave_max_pos) {  // wave-uniform: some row of this wave sees the tile
+            if (key0 + kKTile - 1 <= wave_min_pos) {  // every row sees every key (and all keys < kv_len)
+                tile_body(std::false_type{}, buf, key0);
+            } else {
+                tile_body(std::true_type{}, buf, key0);
+            }
+        }
+        stage_tile(buf ^ 1);                          // the other buffer: last read one iteration ago
+        __syncthreads();
+    }
+    {   // the last tile holds the workgroup's diagonal: never fully visible to a wave
+        const int it = num_tiles - 1;
+        const int key0 = it * kKTile;
+        if (wave_has_rows && key0 <= wave_max_pos) tile_body(std::true_type{}, it & 1, key0);
+        __syncthreads();                              // the next part restages buffer 0
     }
 
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-        float l_tot = l_run[u] + __shfl_xor(l_run[u], 16);
-        l_tot += __shfl_xor(l_tot, 32);
+        const float l_tot = lsum[u][0];
         if (my_row[u] < len) {
             const float inv = 1.f / l_tot;
             __half* op = a.o + ((start + my_row[u]) * Hq + hq) * kPD;
@@ -291,6 +343,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
             }
         }
     }
+  }   // part
 }
 
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
@@ -299,7 +352,7 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
     args.num_seqs = num_seqs;
     args.num_q_tiles = cdiv(max_len, kQTile);
     const int64_t pairs8 = ((int64_t)a.num_q_heads * num_seqs + 7) / 8 * 8;     // pairs padded to the XCD count
-    dim3 grid((unsigned)(pairs8 * args.num_q_tiles));
+    dim3 grid((unsigned)(pairs8 * ((args.num_q_tiles + 1) / 2)));
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
@@ -328,6 +381,7 @@ int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
     MKV_REQUIRE(num_kv_heads > 0 && num_q_heads > 0 && num_q_heads % num_kv_heads == 0,
                 "num_q_heads %d must be a multiple of num_kv_heads %d", num_q_heads, num_kv_heads);
     MKV_REQUIRE(num_seqs <= 65535 && num_q_heads <= 65535, "grid dimension limit");
+    MKV_REQUIRE(softmax_scale > 0.f, "softmax_scale must be positive");
     MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0 &&
                     ((uintptr_t)o & 7) == 0,
                 "q/k/v must be 16-byte aligned, o 8-byte aligned");
@@ -360,6 +414,7 @@ int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
     MKV_REQUIRE(num_q_heads > 0 && num_q_heads % pool->num_kv_heads == 0,
                 "num_q_heads %d must be a multiple of num_kv_heads %d", num_q_heads, pool->num_kv_heads);
     MKV_REQUIRE(num_seqs <= 65535 && num_q_heads <= 65535, "grid dimension limit");
+    MKV_REQUIRE(softmax_scale > 0.f, "softmax_scale must be positive");
     MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)o & 7) == 0,
                 "q must be 16-byte aligned, o 8-byte aligned");
     mkv::PrefillArgs a = {};
