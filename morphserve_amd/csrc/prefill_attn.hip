@@ -131,11 +131,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int r0w = q0 + wave * (16 * kU);
     const int wave_min_pos = prefix + r0w;
     const int wave_max_pos = prefix + min(len - 1, r0w + 16 * kU - 1);   // < wave_min_pos: no row at all
-    int my_row[kU], my_pos[kU];
+    int my_row[kU], my_last_key[kU];   // a row sees keys 0 .. its own position (and < kv_len)
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
         my_row[u] = r0w + u * 16 + m;
-        my_pos[u] = prefix + my_row[u];
+        my_last_key[u] = min(prefix + my_row[u], kv_len - 1);
     }
 
     // Q^T as B operand: lane (row m, group c) holds dims c*32 + 8x .. +8 for product x
@@ -177,14 +177,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     // global -> registers for one 64-key tile: 16 bytes per thread per step.  Keys at or past
     // kv_len re-read the last visible key (finite values; their scores are masked and their
     // probabilities are zero); unmapped table entries read as zeros.
+    // Contiguous source: one uniform base per (sequence, kv head) plus a 32-bit byte offset
+    // per lane that advances by a constant per tile (the launcher bounds len * Hkv * 256).
     v4u kreg[kFetchSteps], vreg[kFetchSteps];
+    const uint32_t row_stride = (uint32_t)Hkv * (kPD * 2);
+    const char* k_src = PAGED ? nullptr : (const char*)a.k + (start * Hkv + kvh) * (int64_t)(kPD * 2);
+    const char* v_src = PAGED ? nullptr : (const char*)a.v + (start * Hkv + kvh) * (int64_t)(kPD * 2);
+    const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + (tid & 15) * 16;
+    uint32_t next_off = (uint32_t)(tid >> 4) * row_stride + (tid & 15) * 16;     // key (tid >> 4) of the next tile
     auto fetch_tile = [&](int key0) {
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
-            const int idx = tid + kThreads * u;
-            const int ch = idx & 15;
-            const int pos = min(key0 + (idx >> 4), kv_len - 1);
             if (PAGED) {
+                const int idx = tid + kThreads * u;
+                const int ch = idx & 15;
+                const int pos = min(key0 + (idx >> 4), kv_len - 1);
                 const int64_t pid = bt_row[pos / pool.block_size];
                 kreg[u] = (v4u){0u, 0u, 0u, 0u};
                 vreg[u] = kreg[u];
@@ -196,18 +203,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                     vreg[u] = *(const v4u*)(ba.v + off);
                 }
             } else {
-                const int64_t off = ((start + pos) * Hkv + kvh) * kPD + ch * 8;
-                kreg[u] = *(const v4u*)(a.k + off);
-                vreg[u] = *(const v4u*)(a.v + off);
+                const uint32_t off = min(next_off + (uint32_t)u * 16u * row_stride, last_off);
+                kreg[u] = *(const v4u*)(k_src + off);
+                vreg[u] = *(const v4u*)(v_src + off);
             }
         }
+        next_off += kKTile * row_stride;
     };
+    const int k_wr_off = (tid >> 4) * kRowBytes + (tid & 15) * 16;           // + 16u rows
+    const int v_wr_off = (tid >> 4) * kRowBytesV + (tid & 15) * 16;
     auto stage_tile = [&](int buf) {
+        char* kw = k_lds + buf * kKBuf + k_wr_off;
+        char* vw = v_lds + buf * kVBuf + v_wr_off;
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
-            const int idx = tid + kThreads * u;
-            *(v4u*)(k_lds + buf * kKBuf + (idx >> 4) * kRowBytes + (idx & 15) * 16) = kreg[u];
-            *(v4u*)(v_lds + buf * kVBuf + (idx >> 4) * kRowBytesV + (idx & 15) * 16) = vreg[u];
+            *(v4u*)(kw + u * (kThreads / 16) * kRowBytes) = kreg[u];
+            *(v4u*)(vw + u * (kThreads / 16) * kRowBytesV) = vreg[u];
         }
     };
 
@@ -220,6 +231,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const char* k_rd = k_lds + buf * kKBuf + k_rd_off;
         const char* v_rd = v_lds + buf * kVBuf + v_rd_off;
         // ---- raw scores of the four 16-key sub-tiles, both column tiles ------------------
+        // (matrix phases run at raised wave priority: the SIMD's other wave fills the gaps with
+        // its softmax arithmetic instead of competing for the matrix pipe in lockstep)
+        __builtin_amdgcn_s_setprio(2);
         // K fragments of sub-tile n+1 are requested before the products of sub-tile n, so
         // the LDS latency is covered by eight matrix instructions
         v4f st[kU][4];
@@ -250,11 +264,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const int key_pos = key0 + 16 * n + 4 * c + j;
-                        if (!(key_pos <= my_pos[u] && key_pos < kv_len)) st[u][n][j] = kPNegBig;
+                        if (key_pos > my_last_key[u]) st[u][n][j] = kPNegBig;
                     }
             }
         }
         // ---- online softmax per column tile -----------------------------------------------
+        __builtin_amdgcn_s_setprio(0);
         v8h pb[kU][2];                 // P^T as B operand: [pair of sub-tiles] = 8 k-slots
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
@@ -283,6 +298,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                                  (_Float16)p[2 * h + 1][2], (_Float16)p[2 * h + 1][3]};
         }
         // ---- O^T += V^T . P^T, 32 keys per product ----------------------------------------
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const char* vp = v_rd + 32 * h * kRowBytesV;
@@ -301,6 +317,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                     acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][h], acc[u][t], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
     };
 
     const int num_tiles = (kv_len + kKTile - 1) / kKTile;
@@ -382,6 +399,7 @@ int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
                 "num_q_heads %d must be a multiple of num_kv_heads %d", num_q_heads, num_kv_heads);
     MKV_REQUIRE(num_seqs <= 65535 && num_q_heads <= 65535, "grid dimension limit");
     MKV_REQUIRE(softmax_scale > 0.f, "softmax_scale must be positive");
+    MKV_REQUIRE((int64_t)max_len * num_kv_heads < (1 << 23), "max_len * num_kv_heads must be below 2^23");
     MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0 &&
                     ((uintptr_t)o & 7) == 0,
                 "q/k/v must be 16-byte aligned, o 8-byte aligned");
