@@ -57,6 +57,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ctx", type=int, nargs=2, default=[1024, 1536], metavar=("LO", "HI"),
                     help="decode workloads: context lengths are uniform in [LO, HI] (at most 2048)")
+    ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
+                    help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
+                         "benchmark's definition) or in id order (diagnostic only)")
     ap.add_argument("--seed", type=int, default=2)
     return ap.parse_args()
 
@@ -93,6 +96,8 @@ def bench_decode(args):
 
     # block tables: a seeded permutation of the whole pool dealt in order
     perm = rng.permutation(num_blocks)
+    if args.tables == "identity":                 # diagnostic: blocks in id order, no gather scatter
+        perm = np.arange(num_blocks)
     seq_ids = rng.permutation(max_seqs)[:N].astype(np.int32)
     table = np.full((max_seqs, max_blocks_per_seq), -1, dtype=np.int32)
     pos = 0
@@ -229,7 +234,7 @@ def bench_decode(args):
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {L} layers, GQA {HQ}q/{HKV}kv, head_dim 128, block 16, "
                                f"batch {N}, ctx U[{args.ctx[0]},{args.ctx[1]}], pool {num_blocks} blocks "
-                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), permuted tables",
+                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), {args.tables} tables",
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
                    "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},
