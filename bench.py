@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "cfg4_mixed", "copy_calibration"])
+                             "cfg4_mixed", "copy_calibration", "eviction"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -503,6 +503,81 @@ def bench_copy_calibration(args):
             "bytes_read_per_launch": moved, "bytes_written_per_launch": moved}
 
 
+# ---------------------------------------------------------------------------------
+def bench_eviction(args):
+    """Swap sequences out to host swap space and back (config-2 block geometry, 2 MiB per
+    block): whole ``_swap`` calls -- block-manager work, copy, synchronisation -- as PCIe GB/s."""
+    import torch
+    from morphserve_amd import ElasticKVPool, KVSwapper, _capi
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    small = _eviction_routes(args, 1, 32, args.pool_blocks or 8192, 32, 40)     # config-1 geometry: 256 KiB blocks
+    torch.cuda.empty_cache()
+    results, gbytes, n_seq, blocks_per_seq, num_blocks = _eviction_routes(args, 32, 8, args.pool_blocks or 4096, 16, 80)
+    best = results["kernel_pinned"]
+    return {
+        "metric": "KV eviction (swap out + swap in of 16 sequences), PCIe GB/s, 1 MI355X",
+        "value": round(2 * gbytes / ((best["swap_out_ms"] + best["swap_in_ms"]) * 1e-3), 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(best["swap_out_ms"] + best["swap_in_ms"], 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"eviction: 2 MiB blocks (K+V), {n_seq} sequences x {blocks_per_seq} scattered blocks "
+                               f"= {gbytes:.2f} GB each way, pool {num_blocks} blocks"},
+        "routes": results,
+        "routes_256KiB_blocks": {"workload": f"{small[2]} sequences x {small[3]} scattered blocks = "
+                                             f"{small[1]:.2f} GB each way", **small[0]},
+        "roofline": None,
+    }
+
+
+def _eviction_routes(args, L, HKV, num_blocks, n_seq, blocks_per_seq):
+    import torch
+    from morphserve_amd import ElasticKVPool, KVSwapper
+    D, B = 128, 16
+    rng = np.random.default_rng(args.seed)
+    pool = ElasticKVPool(num_blocks, L, HKV, B, D, max_seqs_in_block_table=64, max_blocks_per_seq=128,
+                         zero_init=False)
+    bm = pool.block_manager
+    # scattered ownership: blocks dealt from a permutation of the pool
+    perm = rng.permutation(num_blocks)[:n_seq * blocks_per_seq]
+    table = np.full(tuple(bm.block_table.shape), -1, dtype=np.int32)
+    for s_ in range(n_seq):
+        table[s_, :blocks_per_seq] = perm[s_ * blocks_per_seq:(s_ + 1) * blocks_per_seq]
+    bm.block_table.copy_(torch.from_numpy(table))
+    bm.num_seq_allocated_blocks[:n_seq] = blocks_per_seq
+    free = np.ones(num_blocks, dtype=bool)
+    free[perm] = False
+    bm.is_block_free.copy_(torch.from_numpy(free))
+    bm.num_free_blocks = int(free.sum())
+    seqs = list(range(n_seq))
+    moved = n_seq * blocks_per_seq
+    gbytes = moved * pool.block_bytes * 2 / 1e9
+    results = {}
+    for name, pinned, use_kernel in (("kernel_pinned", True, True), ("memcpy_runs_pinned", True, False),
+                                     ("memcpy_runs_pageable", False, False)):
+        sw = KVSwapper(pool, moved + 64, pinned=pinned)
+        out_ms, in_ms = [], []
+        for rep in range(max(args.warmup, 1) + args.steps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            sw.swap_out_seqs(seqs, use_kernel=use_kernel)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            sw.swap_in_seqs(seqs, use_kernel=use_kernel)
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            if rep >= max(args.warmup, 1):
+                out_ms.append((t1 - t0) * 1e3)
+                in_ms.append((t2 - t1) * 1e3)
+        results[name] = {"swap_out_ms": round(float(np.mean(out_ms)), 3), "swap_in_ms": round(float(np.mean(in_ms)), 3),
+                         "swap_out_GBs": round(gbytes / (np.mean(out_ms) * 1e-3), 2),
+                         "swap_in_GBs": round(gbytes / (np.mean(in_ms) * 1e-3), 2)}
+        del sw
+    del pool
+    return results, gbytes, n_seq, blocks_per_seq, num_blocks
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -517,7 +592,7 @@ def main():
     _capi.lib()
     out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
            "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
-           "copy_calibration": bench_copy_calibration}[args.workload](args)
+           "copy_calibration": bench_copy_calibration, "eviction": bench_eviction}[args.workload](args)
     print(json.dumps(out))
 
 

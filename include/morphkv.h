@@ -251,6 +251,18 @@ int mkv_swap_blocks(const int64_t* src_ids, const int64_t* dst_ids, int64_t coun
                     int32_t is_swap_in, const mkv_pool* pool, void* k_swap,
                     void* v_swap, int64_t* num_copies, void* stream);
 
+/* The same eviction with the id lists left on the DEVICE (what
+ * gather_allocated_blocks_and_free / allocate_blocks_for_seqs return,
+ * MS/worker/model.py:476-477, before the reference's .tolist() at :483-484) and
+ * the swap space in PINNED host memory: one kernel moves every pair over PCIe,
+ * scattered or not, with no host synchronisation.  Pairs naming a block outside
+ * the pool or outside [0, num_host_blocks) are skipped.  Replaces the memcpy
+ * loops of CS/block_swapping.cpp:40-84, :120-200 for callers that pin their
+ * swap space (the reference's is pageable, MS/worker/model.py:203-204). */
+int mkv_swap_blocks_device_ids(const int64_t* src_ids, const int64_t* dst_ids, int64_t count,
+                               int32_t is_swap_in, const mkv_pool* pool, void* k_swap,
+                               void* v_swap, int64_t num_host_blocks, void* stream);
+
 /* ---- measurement ---------------------------------------------------------- */
 /* Kernel ids for mkv_prof_*. */
 #define MKV_K_APPEND_DECODE   0
@@ -260,7 +272,8 @@ int mkv_swap_blocks(const int64_t* src_ids, const int64_t* dst_ids, int64_t coun
 #define MKV_K_MIGRATE         4
 #define MKV_K_PREFILL_ATTN    5
 #define MKV_K_FILL_ZERO       6
-#define MKV_K_COUNT           7
+#define MKV_K_SWAP            7
+#define MKV_K_COUNT           8
 /* When enabled, every launch of the kernels above is bracketed by a
  * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
  * returns the launch count and summed duration since the last reset. */

@@ -10,6 +10,8 @@ Drop-in names (reference file each mirrors):
 * ``worker.infer_state.LlamaInferState``             MorphServe/worker/infer_state.py
 * ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
 * ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
+* ``worker.swap.KVSwapper``                          MorphServe/worker/model.py:468-534 (sequence eviction)
+* ``server.Scheduler``                               MorphServe/server/scheduler.py
 
 All compute goes through ``libmorphkv.so`` (hand-written HIP for gfx950) via
 ctypes; nothing here falls back to eager PyTorch.
@@ -21,4 +23,5 @@ from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
 from .worker.kernels.paged_attn import decode_append_and_attend, paged_attention  # noqa: F401
 from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401
 from .elastic_pool import ElasticKVPool  # noqa: F401
+from .worker.swap import KVSwapper  # noqa: F401
 from . import swiftllm_c  # noqa: F401

@@ -16,7 +16,7 @@ MKV_OK, MKV_EINVAL, MKV_EHIP, MKV_ENOSPC, MKV_ELOGIC = 0, -1, -2, -3, -4
 MKV_MAX_SEGMENTS = 128
 
 K_APPEND_DECODE, K_APPEND_PREFILL, K_ATTN_PHASE1, K_ATTN_PHASE2 = 0, 1, 2, 3
-K_MIGRATE, K_PREFILL_ATTN, K_FILL_ZERO = 4, 5, 6
+K_MIGRATE, K_PREFILL_ATTN, K_FILL_ZERO, K_SWAP = 4, 5, 6, 7
 
 
 class MkvPool(C.Structure):
@@ -70,6 +70,7 @@ PROTOTYPES = {
     "mkv_pool_migrate": [_PP, _P, _P, _I64, _P],
     "mkv_bt_remap": [_P, _I64, _P, _I64, _P, _I64, _P],
     "mkv_swap_blocks": [_P, _P, _I64, _I32, _PP, _P, _P, C.POINTER(_I64), _P],
+    "mkv_swap_blocks_device_ids": [_P, _P, _I64, _I32, _PP, _P, _P, _I64, _P],
     "mkv_prof_enable": [_I32],
     "mkv_prof_reset": [],
     "mkv_prof_collect": [_I32, C.POINTER(_I64), C.POINTER(C.c_double)],

@@ -51,6 +51,49 @@ __global__ __launch_bounds__(kCopyThreads) void pool_migrate_kernel(
     }
 }
 
+// Eviction without the host in the loop: the (device block, host block) pairs are
+// read from DEVICE arrays and one launch moves every pair between the pool and a
+// pinned host swap space that the GPU addresses directly over PCIe.  Same item
+// decomposition as the migration kernel; scattered pairs cost nothing extra.
+template <bool SWAP_IN>
+__global__ __launch_bounds__(kCopyThreads) void pool_swap_kernel(
+    const mkv_pool pool, const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
+    int64_t count, char* __restrict__ k_swap, char* __restrict__ v_swap, int64_t num_host_blocks,
+    int64_t block_bytes, int32_t chunks_per_block) {
+    const int64_t total_blocks = pool_total_blocks(pool);
+    const int64_t items = count * 2 * chunks_per_block;
+    for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
+        const int64_t mv = w / (2 * chunks_per_block);
+        const int rem = (int)(w - mv * 2 * chunks_per_block);
+        const int is_v = rem / chunks_per_block;
+        const int chunk = rem - is_v * chunks_per_block;
+        const int64_t dev_id = SWAP_IN ? dst[mv] : src[mv];
+        const int64_t host_id = SWAP_IN ? src[mv] : dst[mv];
+        if (dev_id < 0 || dev_id >= total_blocks || host_id < 0 || host_id >= num_host_blocks) continue;
+        BlockAddr da = block_addr(pool, dev_id, block_bytes);
+        const int64_t off = (int64_t)chunk * kChunkBytes;
+        char* dev_p = const_cast<char*>(is_v ? da.v : da.k) + off;
+        char* host_p = (is_v ? v_swap : k_swap) + host_id * block_bytes + off;
+        const uint4* sp = (const uint4*)(SWAP_IN ? host_p : dev_p) + threadIdx.x;
+        uint4* dp = (uint4*)(SWAP_IN ? dev_p : host_p) + threadIdx.x;
+        const int64_t left = block_bytes - off;
+        if (left >= kChunkBytes) {
+            v4u r[kCopyUnroll];
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) r[u] = __builtin_nontemporal_load((const v4u*)sp + u * kCopyThreads);
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(r[u], (v4u*)dp + u * kCopyThreads);
+        } else {
+            const int64_t units = left >> 4;
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) {
+                const int64_t idx = (int64_t)u * kCopyThreads + threadIdx.x;
+                if (idx < units) dp[u * kCopyThreads] = sp[u * kCopyThreads];
+            }
+        }
+    }
+}
+
 // One 16-byte store per thread, one 4 KiB run per workgroup, plain (cached) stores:
 // on this part that shape writes fastest (a persistent grid-stride loop or
 // non-temporal stores are 15-25 % slower).
@@ -180,6 +223,51 @@ int mkv_swap_blocks(const int64_t* src_ids, const int64_t* dst_ids, int64_t coun
         i = j;
     }
     if (num_copies) *num_copies = copies;
+    return MKV_OK;
+}
+
+int mkv_swap_blocks_device_ids(const int64_t* src_ids, const int64_t* dst_ids, int64_t count,
+                               int32_t is_swap_in, const mkv_pool* pool, void* k_swap, void* v_swap,
+                               int64_t num_host_blocks, void* stream) {
+    int rc = mkv::check_pool(pool);
+    if (rc) return rc;
+    MKV_REQUIRE(count >= 0 && num_host_blocks >= 0, "count/num_host_blocks must be >= 0");
+    if (count == 0) return MKV_OK;
+    MKV_REQUIRE(src_ids && dst_ids && k_swap && v_swap, "NULL argument");
+    // the swap space must be memory the GPU can address: pinned host (or device) memory
+    void* dev_ptr[2] = {nullptr, nullptr};
+    void* host_ptr[2] = {k_swap, v_swap};
+    for (int t = 0; t < 2; ++t) {
+        hipPointerAttribute_t attr;
+        hipError_t e = hipPointerGetAttributes(&attr, host_ptr[t]);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            MKV_REQUIRE(false, "swap space is not pinned host memory (allocate it with hipHostMalloc / pin_memory=True)");
+        }
+        MKV_REQUIRE(attr.type == hipMemoryTypeHost || attr.type == hipMemoryTypeDevice ||
+                        attr.type == hipMemoryTypeManaged,
+                    "swap space is not pinned host memory (allocate it with hipHostMalloc / pin_memory=True)");
+        dev_ptr[t] = attr.devicePointer ? attr.devicePointer : host_ptr[t];
+    }
+    const int64_t block_bytes = mkv::pool_block_bytes(*pool);
+    const int chunks = mkv::cdiv(block_bytes, mkv::kChunkBytes);
+    const int64_t items = count * 2 * chunks;
+    const int64_t want = (int64_t)mkv::num_cus() * 4;
+    const unsigned grid = (unsigned)(items < want ? items : want);
+    hipStream_t s = (hipStream_t)stream;
+    {
+        mkv::ProfScope prof(MKV_K_SWAP, s);
+        if (is_swap_in) {
+            hipLaunchKernelGGL(mkv::pool_swap_kernel<true>, dim3(grid), dim3(mkv::kCopyThreads), 0, s, *pool,
+                               src_ids, dst_ids, count, (char*)dev_ptr[0], (char*)dev_ptr[1], num_host_blocks,
+                               block_bytes, chunks);
+        } else {
+            hipLaunchKernelGGL(mkv::pool_swap_kernel<false>, dim3(grid), dim3(mkv::kCopyThreads), 0, s, *pool,
+                               src_ids, dst_ids, count, (char*)dev_ptr[0], (char*)dev_ptr[1], num_host_blocks,
+                               block_bytes, chunks);
+        }
+    }
+    MKV_HIP(hipGetLastError());
     return MKV_OK;
 }
 

@@ -1,0 +1,85 @@
+"""Sequence eviction: MorphServe/worker/model.py:468-534 (``_swap``, ``swap_in_seqs``,
+``swap_out_seqs``, ``free_seqs_resources``) and the swap space of :195-204.
+
+Flow, as in the reference: block counts of the sequences on the source manager ->
+``gather_allocated_blocks_and_free`` there -> ``allocate_blocks_for_seqs`` on the
+destination manager -> copy block ``src[i]`` to block ``dst[i]``.  Two differences:
+the swap space is PINNED host memory (the reference's is pageable), and the id lists
+never leave the device -- the copy is one kernel reading both lists where the reference
+does ``.tolist()`` twice and issues a memcpy pair per run of consecutive ids.
+``use_kernel=False`` keeps the reference's route (host lists, memcpy runs) for pageable
+swap space.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence
+
+import torch
+
+from .. import _capi, swiftllm_c
+from ..elastic_pool import ElasticKVPool
+from .block_manager import BlockManager
+
+
+class KVSwapper:
+    def __init__(self, pool: ElasticKVPool, num_cpu_blocks: int, cpu_block_manager: Optional[BlockManager] = None,
+                 pinned: bool = True):
+        bm = pool.block_manager
+        self.pool = pool
+        self.gpu_block_manager = bm
+        self.cpu_block_manager = cpu_block_manager or BlockManager(
+            "CPU", num_cpu_blocks, bm.block_table.shape[0], bm.block_table.shape[1], bm.block_size,
+            device=str(pool.device))
+        shape = (num_cpu_blocks, *pool.shape_tail)
+        self.k_swap = torch.zeros(shape, dtype=torch.float16, device="cpu", pin_memory=pinned)
+        self.v_swap = torch.zeros(shape, dtype=torch.float16, device="cpu", pin_memory=pinned)
+        self.pinned = pinned
+        self.block_swap = 0          # blocks moved so far (model.py:478)
+
+    def _swap(self, seq_ids_list: Sequence[int], is_swap_in: bool, use_kernel: Optional[bool] = None) -> int:
+        if use_kernel is None:
+            use_kernel = self.pinned
+        if use_kernel and not self.k_swap.is_pinned():       # before any manager state changes
+            raise ValueError("the one-kernel route needs a pinned swap space (pinned=True)")
+        src_mgr = self.cpu_block_manager if is_swap_in else self.gpu_block_manager
+        dst_mgr = self.gpu_block_manager if is_swap_in else self.cpu_block_manager
+        seq_ids = torch.tensor(list(seq_ids_list), dtype=torch.int32, device=self.pool.device)
+        seq_lengths = src_mgr.get_num_allocated_blocks(seq_ids) * self.gpu_block_manager.block_size
+        src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids)          # int32, sequence-major
+        dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths)     # int64, lowest free ids
+        n = int(src_ids.numel())
+        assert int(dst_ids.numel()) == n
+        self.block_swap += n
+        if n == 0:
+            return 0
+        if use_kernel:
+            desc = self.pool.descriptor()
+            _capi.check(_capi.lib().mkv_swap_blocks_device_ids(
+                src_ids.to(torch.int64).data_ptr(), dst_ids.data_ptr(), n, 1 if is_swap_in else 0,
+                C.byref(desc), self.k_swap.data_ptr(), self.v_swap.data_ptr(), self.k_swap.shape[0],
+                _capi.current_stream()))
+            # the temporaries above must outlive the launch; the stream is the caller's
+            torch.cuda.current_stream().synchronize()
+        else:
+            desc = self.pool.descriptor()
+            cnt = C.c_int64(0)
+            src_l, dst_l = src_ids.tolist(), dst_ids.tolist()
+            _capi.check(_capi.lib().mkv_swap_blocks(
+                swiftllm_c._ids(src_l), swiftllm_c._ids(dst_l), n, 1 if is_swap_in else 0, C.byref(desc),
+                self.k_swap.data_ptr(), self.v_swap.data_ptr(), C.byref(cnt), _capi.current_stream()))
+            torch.cuda.current_stream().synchronize()
+        return n
+
+    def swap_in_seqs(self, seq_ids_list: List[int], use_kernel: Optional[bool] = None) -> int:
+        """CPU swap space -> GPU pool for the given sequences."""
+        return self._swap(seq_ids_list, True, use_kernel)
+
+    def swap_out_seqs(self, seq_ids_list: List[int], use_kernel: Optional[bool] = None) -> int:
+        """GPU pool -> CPU swap space for the given sequences."""
+        return self._swap(seq_ids_list, False, use_kernel)
+
+    def free_seqs_resources(self, seq_ids_list: List[int]) -> None:
+        seq_ids = torch.tensor(list(seq_ids_list), dtype=torch.int32, device=self.pool.device)
+        self.gpu_block_manager.free_blocks_for_seqs(seq_ids)
+        self.cpu_block_manager.free_blocks_for_seqs(seq_ids)
