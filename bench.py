@@ -449,6 +449,33 @@ def bench_mixed(args):
         avg[name] = ms / cnt if cnt else None
     _capi.prof_enable(False)
     _capi.prof_reset()
+
+    # the step before the append: rotary embedding of q and k, separate or fused with it
+    from morphserve_amd import rotary_embedding_and_store_kvcache, rotary_embedding_inplace, rotary_tables
+    cos_t, sin_t = rotary_tables(D, 4096, device="cuda")
+    positions = np.concatenate([np.arange(n) for n in p_lens] + [np.asarray(d_lens) - 1])
+    pos_t = torch.from_numpy(positions).to(dev)
+    st.position_cos, st.position_sin = cos_t[pos_t].contiguous(), sin_t[pos_t].contiguous()
+
+    def timed(fn, reps=20):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def rope_then_store():
+        rotary_embedding_inplace(q, k, st)
+        store_kvcache(k, v, k_cache, v_cache, [], [], bt, model, engine, st, 0)
+
+    rope_two_ms = timed(rope_then_store)
+    rope_fused_ms = timed(lambda: rotary_embedding_and_store_kvcache(q, k, v, k_cache, v_cache, [], [], bt, model,
+                                                                      engine, st, 0))
+    row = D * 2
+    rope_bytes = n_tok * (2 * HQ * row + 2 * HKV * row + HKV * row + 2 * HKV * row + 2 * (D // 2) * 2)
     flops = sum(HQ * 4 * D * (n * n) / 2 for n in p_lens)                  # causal half, QK^T + PV
     tflops = flops / (avg["prefill_attn"] * 1e-3) / 1e12
     append_bytes = 2 * T * 2 * HKV * D * 2
@@ -464,6 +491,8 @@ def bench_mixed(args):
         "prefill_attn_TFLOPs": round(tflops, 1), "prefill_flops_per_layer": flops,
         "append_prefill_GBs": round(append_bytes / (avg["append_prefill"] * 1e-3) / 1e9, 1),
         "decode_attn_GBs": round(dec_bytes / (avg["attn_phase1"] * 1e-3) / 1e9, 1),
+        "rotary_then_store_ms": round(rope_two_ms, 5), "rotary_store_fused_ms": round(rope_fused_ms, 5),
+        "rotary_store_fused_GBs": round(rope_bytes / (rope_fused_ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false>", "achieved": round(tflops, 1),
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4), "traffic": None},
     }

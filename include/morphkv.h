@@ -240,6 +240,27 @@ int mkv_bt_remap(int32_t* block_table, int64_t max_blocks_per_seq,
                  const int32_t* num_seq_allocated_blocks, int64_t max_seqs,
                  const int32_t* remap, int64_t num_blocks, void* stream);
 
+/* ---- rotary embedding, optionally fused with the append --------------------- */
+/* rotary_embedding_inplace, MS/worker/kernels/rotary_emb.py:7-58: q [T, Hq, D] and
+ * k [T, Hkv, D] are rotated in place with row t of cos / sin [T, D/2] (all fp16;
+ * pairs are (d, d + D/2)).  With store != 0 the same launch also does what
+ * store_kvcache does next (MS/worker/layers/transformer_layer.py:93-126,
+ * kvcache_mgmt.py:321-343): the rotated k row and the v row of every token are
+ * written to the token's cache slot -- prefill rows t < num_prefill_tokens at
+ * position t - start of their sequence, decode rows at position len - 1; row
+ * arguments as for mkv_append_prefill / mkv_append_decode, seq_ids holding the
+ * prefill sequences first.  With store == 0 pool, v and the row arguments are
+ * ignored. */
+int mkv_rope_store_kvcache(void* q, void* k, const void* v, const void* cos_table,
+                           const void* sin_table, const mkv_pool* pool,
+                           const int32_t* block_table, int64_t max_blocks_per_seq,
+                           const int32_t* seq_ids, const int32_t* prefill_start_locs,
+                           const int32_t* prefill_lens, const int32_t* decoding_seq_lens,
+                           int32_t num_prefill_seqs, int32_t num_prefill_tokens,
+                           int32_t num_decoding_seqs, int32_t num_q_heads,
+                           int32_t num_kv_heads, int32_t head_dim, int32_t layer,
+                           int32_t store, void* stream);
+
 /* ---- eviction ------------------------------------------------------------ */
 /* swap_blocks / swap_blocks_new_kv_combined, CS/block_swapping.cpp:22-85,
  * :88-202.  src_ids/dst_ids are HOST arrays; k_swap/v_swap are HOST tensors
@@ -273,7 +294,8 @@ int mkv_swap_blocks_device_ids(const int64_t* src_ids, const int64_t* dst_ids, i
 #define MKV_K_PREFILL_ATTN    5
 #define MKV_K_FILL_ZERO       6
 #define MKV_K_SWAP            7
-#define MKV_K_COUNT           8
+#define MKV_K_ROPE_STORE      8
+#define MKV_K_COUNT           9
 /* When enabled, every launch of the kernels above is bracketed by a
  * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
  * returns the launch count and summed duration since the last reset. */

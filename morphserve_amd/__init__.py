@@ -5,6 +5,7 @@ Drop-in names (reference file each mirrors):
 * ``worker.kernels.kvcache_mgmt.store_kvcache``      MorphServe/worker/kernels/kvcache_mgmt.py
 * ``worker.kernels.paged_attn.paged_attention``      MorphServe/worker/kernels/paged_attn.py
 * ``worker.kernels.prefill_attn.prefill_attention``  MorphServe/worker/kernels/prefill_attn.py
+* ``worker.kernels.rotary_emb.*``                    MorphServe/worker/kernels/rotary_emb.py (+ fused append)
 * ``worker.kernels.block_mgmt.*``                    MorphServe/worker/kernels/block_mgmt.py
 * ``worker.block_manager.BlockManager``              MorphServe/worker/block_manager.py
 * ``worker.infer_state.LlamaInferState``             MorphServe/worker/infer_state.py
@@ -22,6 +23,8 @@ from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
 from .worker.kernels.paged_attn import decode_append_and_attend, paged_attention  # noqa: F401
 from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401
+from .worker.kernels.rotary_emb import (rotary_embedding_and_store_kvcache, rotary_embedding_inplace,  # noqa: F401
+                                        rotary_tables)
 from .elastic_pool import ElasticKVPool  # noqa: F401
 from .worker.swap import KVSwapper  # noqa: F401
 from . import swiftllm_c  # noqa: F401

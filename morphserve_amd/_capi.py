@@ -16,7 +16,7 @@ MKV_OK, MKV_EINVAL, MKV_EHIP, MKV_ENOSPC, MKV_ELOGIC = 0, -1, -2, -3, -4
 MKV_MAX_SEGMENTS = 128
 
 K_APPEND_DECODE, K_APPEND_PREFILL, K_ATTN_PHASE1, K_ATTN_PHASE2 = 0, 1, 2, 3
-K_MIGRATE, K_PREFILL_ATTN, K_FILL_ZERO, K_SWAP = 4, 5, 6, 7
+K_MIGRATE, K_PREFILL_ATTN, K_FILL_ZERO, K_SWAP, K_ROPE_STORE = 4, 5, 6, 7, 8
 
 
 class MkvPool(C.Structure):
@@ -69,6 +69,8 @@ PROTOTYPES = {
     "mkv_pool_plan_shrink": [_P, _I64, _I64, _P, _P, _I64, _P, _P, _P],
     "mkv_pool_migrate": [_PP, _P, _P, _I64, _P],
     "mkv_bt_remap": [_P, _I64, _P, _I64, _P, _I64, _P],
+    "mkv_rope_store_kvcache": [_P, _P, _P, _P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32,
+                               _I32, _I32, _I32, _P],
     "mkv_swap_blocks": [_P, _P, _I64, _I32, _PP, _P, _P, C.POINTER(_I64), _P],
     "mkv_swap_blocks_device_ids": [_P, _P, _I64, _I32, _PP, _P, _P, _I64, _P],
     "mkv_prof_enable": [_I32],

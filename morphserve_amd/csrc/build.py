@@ -20,6 +20,7 @@ LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = [
     "core.hip",
     "kv_append.hip",
+    "rope.hip",
     "paged_attn_decode.hip",
     "prefill_attn.hip",
     "block_pool.hip",
