@@ -60,6 +60,9 @@ def parse_args():
     ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
                     help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
                          "benchmark's definition) or in id order (diagnostic only)")
+    ap.add_argument("--pool-backing", choices=["torch", "vmm"], default="torch",
+                    help="decode workloads: the pool is a torch allocation (default) or one tensor over HIP "
+                         "virtual memory (VmmKVPool)")
     ap.add_argument("--seed", type=int, default=2)
     return ap.parse_args()
 
@@ -107,8 +110,13 @@ def bench_decode(args):
     live = perm[:pos].copy()
 
     shape = (num_blocks, L, HKV, B, D)
-    k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
-    v_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+    if args.pool_backing == "vmm":                # one tensor over HIP virtual memory, 64-block chunks
+        from morphserve_amd import VmmKVPool
+        vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, chunk_blocks=64)
+        k_cache, v_cache = vmm_pool.k_cache, vmm_pool.v_cache
+    else:
+        k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+        v_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     live_t = torch.from_numpy(live).to(dev)
@@ -234,7 +242,8 @@ def bench_decode(args):
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {L} layers, GQA {HQ}q/{HKV}kv, head_dim 128, block 16, "
                                f"batch {N}, ctx U[{args.ctx[0]},{args.ctx[1]}], pool {num_blocks} blocks "
-                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), {args.tables} tables",
+                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), {args.tables} tables"
+                               + (", pool over HIP virtual memory" if args.pool_backing == "vmm" else ""),
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
                    "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},

@@ -240,6 +240,23 @@ int mkv_bt_remap(int32_t* block_table, int64_t max_blocks_per_seq,
                  const int32_t* num_seq_allocated_blocks, int64_t max_seqs,
                  const int32_t* remap, int64_t num_blocks, void* stream);
 
+/* ---- pool backing through virtual memory ---------------------------------- */
+/* Where the reference grows the pool with tensor views over freed weight memory
+ * (acquire_new_kvcache, CS/memory_manager.cpp:69-176) and drops them again
+ * (free_kv_cache_tensors, MS/server/memory_utils.py:602-610), an arena reserves
+ * reserve_bytes of device ADDRESS space once and maps physical chunks of
+ * chunk_bytes at its end: a pool built on it is one contiguous
+ * [num_blocks, L, Hkv, B, D] tensor at a fixed address whatever its size, with
+ * no extension segments.  mkv_arena_resize maps or unmaps whole chunks at the
+ * end (host call; the caller makes sure no kernel still uses memory it gives
+ * back); MKV_ENOSPC when the device has no memory left (nothing changed). */
+typedef struct mkv_arena mkv_arena;
+int mkv_arena_create(uint64_t reserve_bytes, uint64_t chunk_bytes, mkv_arena** out);
+int mkv_arena_info(const mkv_arena* arena, void** base, uint64_t* reserved_bytes,
+                   uint64_t* chunk_bytes, uint64_t* mapped_bytes);
+int mkv_arena_resize(mkv_arena* arena, uint64_t mapped_bytes);
+int mkv_arena_destroy(mkv_arena* arena);
+
 /* ---- rotary embedding, optionally fused with the append --------------------- */
 /* rotary_embedding_inplace, MS/worker/kernels/rotary_emb.py:7-58: q [T, Hq, D] and
  * k [T, Hkv, D] are rotated in place with row t of cos / sin [T, D/2] (all fp16;

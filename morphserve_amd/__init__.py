@@ -11,6 +11,7 @@ Drop-in names (reference file each mirrors):
 * ``worker.infer_state.LlamaInferState``             MorphServe/worker/infer_state.py
 * ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
 * ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
+* ``vmm_pool.VmmKVPool``                             the same pool as ONE tensor over HIP virtual memory
 * ``worker.swap.KVSwapper``                          MorphServe/worker/model.py:468-534 (sequence eviction)
 * ``server.Scheduler``                               MorphServe/server/scheduler.py
 
@@ -26,5 +27,6 @@ from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_atte
 from .worker.kernels.rotary_emb import (rotary_embedding_and_store_kvcache, rotary_embedding_inplace,  # noqa: F401
                                         rotary_tables)
 from .elastic_pool import ElasticKVPool  # noqa: F401
+from .vmm_pool import VmmKVPool  # noqa: F401
 from .worker.swap import KVSwapper  # noqa: F401
 from . import swiftllm_c  # noqa: F401

@@ -25,6 +25,7 @@ SOURCES = [
     "prefill_attn.hip",
     "block_pool.hip",
     "migrate.hip",
+    "vmm_arena.hip",
 ]
 
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32.

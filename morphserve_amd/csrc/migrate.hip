@@ -147,8 +147,8 @@ int mkv_fill_zero(void* ptr, uint64_t bytes, void* stream) {
     MKV_REQUIRE(ptr != nullptr, "ptr is NULL");
     MKV_REQUIRE(((uintptr_t)ptr & 15) == 0, "ptr must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    // at most 2^30 workgroups (4 TiB) per launch
-    const uint64_t max_bytes = (uint64_t)1 << 42;
+    // a launch may not have 2^32 or more threads: at most 2^31 16-byte units (32 GiB) each
+    const uint64_t max_bytes = (uint64_t)1 << 35;
     char* cur = (char*)ptr;
     while (bytes > 0) {
         const uint64_t now = bytes < max_bytes ? bytes : max_bytes;

@@ -129,6 +129,16 @@ class ElasticKVPool:
         if drop == 0:
             e = torch.empty(0, dtype=torch.int64, device=self.device)
             return e, e
+        src, dst = self._relocate_live_blocks(new_num_blocks)
+        self._drop_segments(drop)
+        return src, dst
+
+    def _relocate_live_blocks(self, new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Plan (device scan) -> batched block copy -> block-table rewrite, then wait: when
+        this returns no live block has an id >= ``new_num_blocks`` and the memory behind
+        those ids is no longer read.  Raises ``RuntimeError`` (state untouched) when the
+        live blocks do not fit below the cut."""
+        bm = self.block_manager
         lib = _capi.lib()
         stream = _capi.current_stream()
         cap = bm.num_blocks - new_num_blocks
@@ -149,7 +159,6 @@ class ElasticKVPool:
                                          bm.num_seq_allocated_blocks.data_ptr(),
                                          bm.num_seq_allocated_blocks.shape[0], remap.data_ptr(),
                                          bm.num_blocks, stream))
-        # the segments must outlive the copy that reads them
+        # the memory above the cut must outlive the copy that reads it
         torch.cuda.current_stream().synchronize()
-        self._drop_segments(drop)
         return src[:moves], dst[:moves]

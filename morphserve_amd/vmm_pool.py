@@ -1,0 +1,154 @@
+"""KV pool backed by HIP virtual memory: one contiguous ``[num_blocks, L, Hkv, B, D]``
+tensor (K, and one for V) that grows and shrinks in place.
+
+The reference grows its pool with extra tensors carved from freed weight memory
+(MorphServe/server/memory_utils.py:369-420) and can only drop the last of them when it
+is empty (:529-544, :617-651); every kernel then needs the segment arithmetic of
+MorphServe/worker/kernels/kvcache_mgmt.py:169-183.  Here the address range of the
+largest pool is reserved once and physical memory is mapped at its end chunk by chunk:
+block ids are plain indices, ``k_cache_new`` stays empty, growing copies nothing, and a
+shrink first relocates the live blocks above the cut (as ``ElasticKVPool.shrink_to``).
+Same ``BlockManager`` and bookkeeping as ``ElasticKVPool``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Tuple
+
+import torch
+
+from . import _capi
+from .elastic_pool import ElasticKVPool
+from .swiftllm_c import _RawDeviceMemory
+from .worker.block_manager import BlockManager
+
+
+class _Arena:
+    def __init__(self, reserve_bytes: int, chunk_bytes: int):
+        self.handle = C.c_void_p()
+        _capi.check(_capi.lib().mkv_arena_create(reserve_bytes, chunk_bytes, C.byref(self.handle)))
+        base = C.c_void_p()
+        _capi.check(_capi.lib().mkv_arena_info(self.handle, C.byref(base), None, None, None))
+        self.base = int(base.value)
+
+    def resize(self, mapped_bytes: int) -> None:
+        rc = _capi.lib().mkv_arena_resize(self.handle, mapped_bytes)
+        if rc == _capi.MKV_ENOSPC:
+            raise MemoryError("the device has no memory left for the pool to grow")
+        _capi.check(rc)
+
+    def mapped_bytes(self) -> int:
+        n = C.c_uint64(0)
+        _capi.check(_capi.lib().mkv_arena_info(self.handle, None, None, None, C.byref(n)))
+        return int(n.value)
+
+    def close(self) -> None:
+        if self.handle:
+            _capi.check(_capi.lib().mkv_arena_destroy(self.handle))
+            self.handle = C.c_void_p()
+
+
+class VmmKVPool(ElasticKVPool):
+    """``num_blocks`` blocks now, room for ``max_blocks``; sizes move in multiples of
+    ``chunk_blocks`` (one physical allocation per chunk and per tensor)."""
+
+    def __init__(self, num_blocks: int, max_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
+                 head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int, chunk_blocks: int = 64,
+                 device: str = "cuda"):
+        _capi.lib()
+        self.device = torch.device(device, torch.cuda.current_device()) if device == "cuda" else torch.device(device)
+        self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
+        self.chunk_blocks = chunk_blocks
+        if num_blocks % chunk_blocks or max_blocks % chunk_blocks or not 0 < num_blocks <= max_blocks:
+            raise ValueError(f"num_blocks and max_blocks must be multiples of chunk_blocks ({chunk_blocks})")
+        self.max_blocks = max_blocks
+        self._k_arena = _Arena(max_blocks * self.block_bytes, chunk_blocks * self.block_bytes)
+        self._v_arena = _Arena(max_blocks * self.block_bytes, chunk_blocks * self.block_bytes)
+        self.k_cache_new, self.v_cache_new = [], []          # never used: the pool is one tensor
+        self.kv_cache_new_block_size = 0
+        self.block_manager = BlockManager("GPU", num_blocks, max_seqs_in_block_table, max_blocks_per_seq,
+                                          block_size, device=device)
+        self._result = torch.zeros(4, dtype=torch.int64, device=device)
+        self._map(num_blocks)
+        self._zero(0, num_blocks)
+
+    # -- mapping ---------------------------------------------------------------------
+    def _map(self, num_blocks: int) -> None:
+        nbytes = num_blocks * self.block_bytes
+        self._k_arena.resize(nbytes)
+        try:
+            self._v_arena.resize(nbytes)
+        except Exception:
+            self._k_arena.resize(self._v_arena.mapped_bytes())
+            raise
+        shape = (num_blocks, *self.shape_tail)
+        self.k_cache = torch.as_tensor(_RawDeviceMemory(self._k_arena.base, shape, self._k_arena), device=self.device)
+        self.v_cache = torch.as_tensor(_RawDeviceMemory(self._v_arena.base, shape, self._v_arena), device=self.device)
+
+    def _zero(self, first: int, count: int) -> None:
+        lib, stream = _capi.lib(), _capi.current_stream()
+        off, nbytes = first * self.block_bytes, count * self.block_bytes
+        _capi.check(lib.mkv_fill_zero(self._k_arena.base + off, nbytes, stream))
+        _capi.check(lib.mkv_fill_zero(self._v_arena.base + off, nbytes, stream))
+
+    def descriptor(self) -> _capi.MkvPool:
+        return _capi.make_pool(self.k_cache, self.v_cache)
+
+    # -- grow / shrink ---------------------------------------------------------------
+    def expand(self, num_new_blocks: int, k_seg=None, v_seg=None) -> None:
+        """Map ``num_new_blocks`` more blocks at the end (zero filled, all free)."""
+        assert k_seg is None and v_seg is None, "a virtual-memory pool maps its own memory"
+        bm = self.block_manager
+        if num_new_blocks <= 0 or num_new_blocks % self.chunk_blocks:
+            raise ValueError(f"the pool grows in multiples of {self.chunk_blocks} blocks")
+        if bm.num_blocks + num_new_blocks > self.max_blocks:
+            raise ValueError(f"at most {self.max_blocks} blocks were reserved")
+        old = bm.num_blocks
+        self._map(old + num_new_blocks)
+        self._zero(old, num_new_blocks)
+        bm.num_blocks += num_new_blocks
+        bm.num_free_blocks += num_new_blocks
+        new_map = torch.empty(bm.num_blocks, dtype=torch.bool, device=self.device)
+        new_map[:old] = bm.is_block_free
+        new_map[old:] = True
+        bm.is_block_free = new_map
+
+    def tail_unused(self, num_blocks: int) -> bool:
+        """True when none of the last ``num_blocks`` blocks is live."""
+        bm = self.block_manager
+        _capi.check(_capi.lib().mkv_bm_count_live(bm.is_block_free.data_ptr(), bm.num_blocks - num_blocks,
+                                                  bm.num_blocks, self._result.data_ptr(), _capi.current_stream()))
+        return int(self._result[0].item()) == 0
+
+    def shrink_to(self, new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Shrink to ``new_num_blocks``: live blocks above the cut move to the lowest free ids
+        below it, the block table is rewritten, the memory above the cut is unmapped.
+        Returns the move lists; raises ``RuntimeError`` (state untouched) when they do not fit."""
+        bm = self.block_manager
+        if not 0 < new_num_blocks <= bm.num_blocks or new_num_blocks % self.chunk_blocks:
+            raise ValueError(f"new size {new_num_blocks} must be a positive multiple of {self.chunk_blocks} "
+                             f"and at most {bm.num_blocks}")
+        removed = bm.num_blocks - new_num_blocks
+        if removed == 0:
+            e = torch.empty(0, dtype=torch.int64, device=self.device)
+            return e, e
+        src, dst = self._relocate_live_blocks(new_num_blocks)        # synchronises the stream
+        bm.num_blocks -= removed
+        bm.num_free_blocks -= removed
+        bm.is_block_free = bm.is_block_free[:new_num_blocks].clone()
+        torch.cuda.synchronize(self.device)                          # nothing may still read the tail
+        self._map(new_num_blocks)
+        return src, dst
+
+    # the segment-based entry points of the parent do not apply
+    def tail_segment_unused(self) -> bool:
+        raise NotImplementedError("a virtual-memory pool has no segments; use tail_unused(num_blocks)")
+
+    def shrink_tail_if_unused(self) -> bool:
+        raise NotImplementedError("a virtual-memory pool has no segments; use shrink_to(num_blocks)")
+
+    def close(self) -> None:
+        """Unmap everything and free the address ranges (the tensors must not be used afterwards)."""
+        self.k_cache = self.v_cache = None
+        self._k_arena.close()
+        self._v_arena.close()

@@ -241,3 +241,22 @@ def test_config4_mixed_batch_one_layer(cuda):
     got = o.cpu().numpy().reshape(n_tok, 32, 128)
     assert_attn_close(got[:T], want_p, "config 4 prefill")
     assert_attn_close(got[T:], want_d, "config 4 decode")
+
+
+def test_zero_fill_larger_than_one_launch(cuda):
+    """40 GiB + 5 bytes: more 16-byte units than one launch may have threads, plus a tail."""
+    from morphserve_amd import _capi
+    if _mem_gib(cuda) < 48:
+        pytest.skip("needs ~41 GiB of free HBM")
+    n = 40 * 2 ** 30 + 5
+    buf = torch.empty(n + 16, dtype=torch.uint8, device=cuda)
+    probes = [0, 1, 2 ** 35 - 1, 2 ** 35, 2 ** 35 + 16, 39 * 2 ** 30 + 7, n - 6, n - 1, n]
+    for p in probes:
+        buf[p] = 0xAB
+    _capi.check(_capi.lib().mkv_fill_zero(buf.data_ptr(), n, _capi.current_stream()))
+    torch.cuda.synchronize()
+    got = [int(buf[p]) for p in probes]
+    assert got == [0] * (len(probes) - 1) + [0xAB], got         # the byte after the range is untouched
+    assert int(buf[:2 ** 31].max()) == 0 and int(buf[n - 2 ** 30:n].max()) == 0
+    sample = buf[:n].view(torch.int64)[::4099] if n % 8 == 0 else buf[:n - 5].view(torch.int64)[::4099]
+    assert int(sample.abs().max()) == 0
