@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "cfg4_mixed", "copy_calibration", "eviction"])
+                             "cfg4_mixed", "cfg5_pressure_shrink", "copy_calibration", "eviction"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -388,6 +388,147 @@ def bench_resize(args):
     }
 
 
+def bench_pressure_shrink(args):
+    """Config 5 as BASELINE states it: CodeLlama-34B-shaped decode on a ~200 GB pool, and
+    mid-run the scheduler's own give-back rule releases 25 % of the blocks (63 578 -> 47 684)
+    while a quarter of the live blocks sit above the cut and have to move."""
+    import torch
+    from morphserve_amd import ElasticKVPool, _capi, build_infer_state, decode_append_and_attend, paged_attention
+    from morphserve_amd.server import PoolEngine, Request, Scheduler
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, HQ, HKV, D, B, N = 48, 64, 8, 128, 16, 128
+    KEEP, SEG = 47684, 15894                       # 63 578 blocks of 3 MiB (K+V) = 186 GiB
+    total = KEEP + SEG
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
+    nblk = (lens.astype(np.int64) + B - 1) // B
+    max_seqs, max_bps = 256, 128
+    pool = ElasticKVPool(KEEP, L, HKV, B, D, max_seqs_in_block_table=max_seqs, max_blocks_per_seq=max_bps)
+    pool.expand(SEG)
+    perm = rng.permutation(total)
+    seq_ids = rng.permutation(max_seqs)[:N].astype(np.int32)
+    table = np.full((max_seqs, max_bps), -1, dtype=np.int32)
+    n_alloc = np.zeros(max_seqs, dtype=np.int32)
+    pos = 0
+    for i in range(N):
+        table[seq_ids[i], :nblk[i]] = perm[pos:pos + nblk[i]]
+        n_alloc[seq_ids[i]] = nblk[i]
+        pos += nblk[i]
+    live = perm[:pos].copy()
+    free = np.ones(total, dtype=bool)
+    free[live] = False
+    bm = pool.block_manager
+    bm.block_table.copy_(torch.from_numpy(table))
+    bm.num_seq_allocated_blocks.copy_(torch.from_numpy(n_alloc))
+    bm.is_block_free.copy_(torch.from_numpy(free))
+    bm.num_free_blocks = int(free.sum())
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    tail = (L, HKV, B, D)
+    for ids, kt, vt, off in ((live[live < KEEP], pool.k_cache, pool.v_cache, 0),
+                             (live[live >= KEEP], pool.k_cache_new[0], pool.v_cache_new[0], KEEP)):
+        idt = torch.from_numpy(ids - off).to(dev)
+        for c0 in range(0, len(ids), 128):
+            idx = idt[c0:c0 + 128]
+            kt[idx] = torch.randn((len(idx), *tail), dtype=torch.float16, device=dev, generator=g)
+            vt[idx] = torch.randn((len(idx), *tail), dtype=torch.float16, device=dev, generator=g)
+    q = torch.randn((L, N, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    k_new = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    v_new = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((L, N, HQ * D), dtype=torch.float16, device=dev)
+    model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
+    ecfg = Cfg(block_size=B, max_blocks_per_seq=max_bps, max_batch_size=256, max_tokens_in_batch=1 << 20,
+               num_cpu_blocks=0, max_seqs_in_block_table=max_seqs, quant_serve=True, num_layers_to_quantize=1,
+               num_layers_to_quantize_max=0)
+
+    def state():
+        return build_infer_state([], seq_ids.tolist(), lens.tolist(), HKV, D, num_blocks_org=bm.num_blocks_org,
+                                 kv_cache_new_block_size=pool.kv_cache_new_block_size)
+
+    def step(st):
+        for layer in range(L):
+            decode_append_and_attend(k_new[layer], v_new[layer], q[layer], pool.k_cache, pool.v_cache,
+                                     pool.k_cache_new, pool.v_cache_new, bm.block_table, model, ecfg, st, layer,
+                                     o[layer])
+
+    def timed_steps(st):
+        for _ in range(max(args.warmup, 1)):
+            step(st)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(st)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    def probe(st):                                  # attention only (no append) on three layers
+        out = torch.empty((3, N, HQ * D), dtype=torch.float16, device=dev)
+        for j, layer in enumerate((0, 17, 47)):
+            paged_attention(q[layer], pool.k_cache, pool.v_cache, pool.k_cache_new, pool.v_cache_new,
+                            bm.block_table, model, ecfg, st, layer, out[j])
+        return out
+
+    st = state()
+    before_ms = timed_steps(st)
+    ref = probe(st)
+
+    # the scheduler decides: running sequences only, nothing waiting, plenty of free blocks
+    engine = PoolEngine(pool, ecfg, num_layers=L, seg_blocks=SEG, migrate=True)
+    engine.model.layer_quant_list.append(L - 1)     # the segment came from replacing the last layer
+    engine.model.is_layer_quant_list[L - 1] = True
+    engine.model.next_unquantized_layer = L - 2
+    sched = Scheduler(model, ecfg, total)
+    engine.scheduler = sched
+    for i in range(N):
+        sched.running_q.append(Request(prompt_len=int(lens[i]) - 1, output_len=1, request_id=int(seq_ids[i])))
+    _capi.prof_reset()
+    _capi.prof_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sched.get_next_batch(engine)
+    torch.cuda.synchronize()
+    shrink_ms = (time.perf_counter() - t0) * 1e3
+    mg_launches, mg_ms = _capi.prof_collect(_capi.K_MIGRATE)
+    _capi.prof_enable(False)
+    _capi.prof_reset()
+    assert pool.num_blocks == KEEP and not pool.k_cache_new and sched.num_gpu_blocks == KEEP, "no give-back happened"
+    moves = engine.migrated_blocks
+    assert moves == int((live >= KEEP).sum())
+
+    st = state()
+    got = probe(st)
+    identical = bool(torch.equal(got, ref))
+    assert identical, "attention outputs changed across the shrink"
+    after_ms = timed_steps(st)
+
+    attn_bytes, append_bytes = decode_bytes_per_layer(lens, N, HQ, HKV, D, B)
+    step_bytes = L * (attn_bytes + append_bytes)
+    moved = moves * 2 * pool.block_bytes
+    return {
+        "metric": "decode step around a pressure-driven pool shrink with live migration, 1 MI355X",
+        "value": round(step_bytes / (after_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(after_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"cfg5_pressure_shrink: 48 layers, GQA 64q/8kv, batch {N}, ctx U[{args.ctx[0]},"
+                               f"{args.ctx[1]}], pool {total} -> {KEEP} blocks of 3 MiB, eager launches"},
+        "ms_per_step_before": round(before_ms, 4), "ms_per_step_after": round(after_ms, 4),
+        "pct_of_hbm_peak_before": round(100 * step_bytes / (before_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "pct_of_hbm_peak_after": round(100 * step_bytes / (after_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "shrink": {"decided_by": "Scheduler.get_next_batch -> try_quant2org -> quant2org_and_update_kvcache(migrate)",
+                   "ms": round(shrink_ms, 3), "live_blocks_moved": moves, "moved_GiB": round(moved / 2 ** 30, 2),
+                   "GBs_read_plus_write": round(2 * moved / (shrink_ms * 1e-3) / 1e9, 1),
+                   "migrate_kernel_ms": round(mg_ms, 3),
+                   "attention_outputs_bit_identical_across_shrink": identical},
+        "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel",
+                     "achieved": round(2 * moved / (mg_ms * 1e-3) / 1e9, 1) if mg_ms else None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(2 * moved / (mg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if mg_ms else None,
+                     "traffic": None},
+    }
+
+
 def bench_mixed(args):
     """Config 4: Llama-2-7B MHA shapes, 32 layers; one step = eight 512-token prefill
     chunks + 120 decode sequences (contexts lognormal(6.2, 0.6) clipped to [16, 768]):
@@ -630,7 +771,8 @@ def main():
     _capi.lib()
     out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
            "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
-           "copy_calibration": bench_copy_calibration, "eviction": bench_eviction}[args.workload](args)
+           "copy_calibration": bench_copy_calibration, "eviction": bench_eviction,
+           "cfg5_pressure_shrink": bench_pressure_shrink}[args.workload](args)
     print(json.dumps(out))
 
 
