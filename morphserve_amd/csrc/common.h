@@ -54,9 +54,10 @@ __device__ __forceinline__ BlockAddr block_addr(const mkv_pool& p, int64_t id, i
         a.k = (const char*)p.k_base + id * block_bytes;
         a.v = (const char*)p.v_base + id * block_bytes;
     } else {
-        int64_t rel = id - p.num_blocks_org;
-        int64_t seg = rel / p.seg_blocks;
-        int64_t local = rel - seg * p.seg_blocks;
+        // ids are below 2^31 (checked with the pool): a 32-bit division, not the 64-bit routine
+        const uint32_t rel = (uint32_t)(id - p.num_blocks_org);
+        const uint32_t seg = rel / (uint32_t)p.seg_blocks;
+        const int64_t local = rel - seg * (uint32_t)p.seg_blocks;
         a.k = (const char*)p.k_seg[seg] + local * block_bytes;
         a.v = (const char*)p.v_seg[seg] + local * block_bytes;
     }

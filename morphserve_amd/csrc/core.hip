@@ -37,6 +37,9 @@ int check_pool(const mkv_pool* p) {
         for (int j = 0; j < p->num_segments; ++j)
             MKV_REQUIRE(p->k_seg[j] && p->v_seg[j], "segment %d has a NULL base", j);
     }
+    MKV_REQUIRE(p->num_blocks_org + (int64_t)p->num_segments * p->seg_blocks <= 0x7fffffff &&
+                    p->seg_blocks <= 0x7fffffff,
+                "block ids are 32-bit: the pool may hold at most 2^31 - 1 blocks");
     MKV_REQUIRE(((uintptr_t)p->k_base & 15) == 0 && ((uintptr_t)p->v_base & 15) == 0,
                 "pool bases must be 16-byte aligned");
     for (int j = 0; j < p->num_segments; ++j)

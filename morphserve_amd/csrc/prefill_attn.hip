@@ -185,22 +185,30 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const char* v_src = PAGED ? nullptr : (const char*)a.v + (start * Hkv + kvh) * (int64_t)(kPD * 2);
     const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + (tid & 15) * 16;
     uint32_t next_off = (uint32_t)(tid >> 4) * row_stride + (tid & 15) * 16;     // key (tid >> 4) of the next tile
+    // Paged source: fetch step u covers keys key0 + 16u .. +15 = ONE block (block_size is 16
+    // here), so its id and address are workgroup-uniform and only the row inside it differs
+    // per thread.  The four ids of a tile are loaded one tile ahead (lane u keeps step u's),
+    // so no fetch ever waits on a table lookup.
+    int32_t tile_ids = 0;
+    auto load_tile_ids = [&](int key0) {
+        if (PAGED) tile_ids = bt_row[min((key0 >> 4) + (lane & 3), (kv_len - 1) >> 4)];
+    };
+    load_tile_ids(0);
     auto fetch_tile = [&](int key0) {
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
             if (PAGED) {
-                const int idx = tid + kThreads * u;
-                const int ch = idx & 15;
-                const int pos = min(key0 + (idx >> 4), kv_len - 1);
-                const int64_t pid = bt_row[pos / pool.block_size];
+                const int blk = min((key0 >> 4) + u, (kv_len - 1) >> 4);
+                const int pos = min(key0 + 16 * u + (tid >> 4), kv_len - 1);
+                const int64_t pid = __builtin_amdgcn_readlane(tile_ids, u);
                 kreg[u] = (v4u){0u, 0u, 0u, 0u};
                 vreg[u] = kreg[u];
                 if (pid >= 0 && pid < total_blocks) {
                     BlockAddr ba = block_addr(pool, pid, block_bytes);
-                    const int64_t off = ((int64_t)a.layer * Hkv + kvh) * ((int64_t)pool.block_size * kPD * 2) +
-                                        (int64_t)(pos % pool.block_size) * (kPD * 2) + ch * 16;
-                    kreg[u] = *(const v4u*)(ba.k + off);
-                    vreg[u] = *(const v4u*)(ba.v + off);
+                    const int64_t head_off = ((int64_t)a.layer * Hkv + kvh) * (int64_t)(16 * kPD * 2);
+                    const uint32_t off = (uint32_t)(pos - (blk << 4)) * (kPD * 2) + (tid & 15) * 16;
+                    kreg[u] = *(const v4u*)(ba.k + head_off + off);
+                    vreg[u] = *(const v4u*)(ba.v + head_off + off);
                 }
             } else {
                 const uint32_t off = min(next_off + (uint32_t)u * 16u * row_stride, last_off);
@@ -209,6 +217,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             }
         }
         next_off += kKTile * row_stride;
+        load_tile_ids(key0 + kKTile);
     };
     const int k_wr_off = (tid >> 4) * kRowBytes + (tid & 15) * 16;           // + 16u rows
     const int v_wr_off = (tid >> 4) * kRowBytesV + (tid & 15) * 16;
@@ -428,6 +437,7 @@ int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
     if (num_seqs == 0 || max_chunk_len == 0) return MKV_OK;
     MKV_REQUIRE(q && o && block_table && seq_ids && start_locs && chunk_lens, "NULL argument");
     MKV_REQUIRE(pool->head_dim == mkv::kPD, "prefill attention supports head_dim 128 only (got %d)", pool->head_dim);
+    MKV_REQUIRE(pool->block_size == 16, "chunked prefill supports block_size 16 only (got %d)", pool->block_size);
     MKV_REQUIRE(layer >= 0 && layer < pool->num_layers, "layer %d outside [0, %d)", layer, pool->num_layers);
     MKV_REQUIRE(num_q_heads > 0 && num_q_heads % pool->num_kv_heads == 0,
                 "num_q_heads %d must be a multiple of num_kv_heads %d", num_q_heads, pool->num_kv_heads);
