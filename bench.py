@@ -624,8 +624,20 @@ def bench_mixed(args):
     rope_two_ms = timed(rope_then_store)
     rope_fused_ms = timed(lambda: rotary_embedding_and_store_kvcache(q, k, v, k_cache, v_cache, [], [], bt, model,
                                                                       engine, st, 0))
+    # chunked prefill over the paged cache: the second 256 tokens of every prompt as a chunk
+    # whose first 256 tokens are already cached (the cache holds the prompts after step())
+    from morphserve_amd import chunked_prefill_attention
+    half = p_lens[0] // 2
+    n_p = len(p_lens)
+    st_chunk = build_infer_state([half] * n_p, seq_ids[:n_p].tolist(), [], HKV, D)
+    q_chunk = torch.randn((n_p * half, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    o_chunk = torch.empty_like(q_chunk)
+    prefix_t = torch.full((n_p,), half, dtype=torch.int32, device=dev)
+    chunk_ms = timed(lambda: chunked_prefill_attention(q_chunk, k_cache, v_cache, [], [], bt, model, engine,
+                                                       st_chunk, 0, o_chunk, prefix_t))
+    chunk_flops = n_p * HQ * 4 * D * (half * half + half * half / 2)
     row = D * 2
-    rope_bytes = n_tok * (2 * HQ * row + 2 * HKV * row + HKV * row + 2 * HKV * row + 2 * (D // 2) * 2)
+    rope_bytes =n_tok * (2 * HQ * row + 2 * HKV * row + HKV * row + 2 * HKV * row + 2 * (D // 2) * 2)
     flops = sum(HQ * 4 * D * (n * n) / 2 for n in p_lens)                  # causal half, QK^T + PV
     tflops = flops / (avg["prefill_attn"] * 1e-3) / 1e12
     append_bytes = 2 * T * 2 * HKV * D * 2
@@ -641,6 +653,9 @@ def bench_mixed(args):
         "prefill_attn_TFLOPs": round(tflops, 1), "prefill_flops_per_layer": flops,
         "append_prefill_GBs": round(append_bytes / (avg["append_prefill"] * 1e-3) / 1e9, 1),
         "decode_attn_GBs": round(dec_bytes / (avg["attn_phase1"] * 1e-3) / 1e9, 1),
+        "chunked_prefill_ms": round(chunk_ms, 5),
+        "chunked_prefill": f"{n_p} chunks of {half} tokens over a {half}-token cached prefix: "
+                           f"{chunk_flops / (chunk_ms * 1e-3) / 1e12:.1f} TFLOP/s",
         "rotary_then_store_ms": round(rope_two_ms, 5), "rotary_store_fused_ms": round(rope_fused_ms, 5),
         "rotary_store_fused_GBs": round(rope_bytes / (rope_fused_ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false>", "achieved": round(tflops, 1),
