@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "cfg4_mixed", "cfg5_pressure_shrink", "copy_calibration", "eviction"])
+                             "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "eviction"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -663,6 +663,144 @@ def bench_mixed(args):
     }
 
 
+def bench_serving(args):
+    """Config 4 as a serving loop on the KV path only (no GEMMs): bursty arrivals (gamma
+    inter-arrival, shape 0.5), 512-token prompts admitted by the scheduler as prefill batches,
+    decode batches in between, sequences finishing at random lengths and freeing their blocks.
+    Every step runs scheduler -> block allocation -> rotary + append -> attention for all 32
+    layers -> frees.  Reports where the time of a step goes."""
+    import torch
+    from morphserve_amd import (ElasticKVPool, build_infer_state, paged_attention, prefill_attention,
+                                rotary_embedding_and_store_kvcache, rotary_tables)
+    from morphserve_amd.server import PoolEngine, Request, Scheduler
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, HQ, HKV, D, B = 32, 32, 32, 128, 16
+    num_blocks = args.pool_blocks or 8192
+    max_seqs, max_bps = 256, 64
+    rng = np.random.default_rng(args.seed)
+    pool = ElasticKVPool(num_blocks, L, HKV, B, D, max_seqs_in_block_table=max_seqs, max_blocks_per_seq=max_bps,
+                         zero_init=False)
+    bm = pool.block_manager
+    model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
+    ecfg = Cfg(block_size=B, max_blocks_per_seq=max_bps, max_batch_size=160, max_tokens_in_batch=8 * 512,
+               num_cpu_blocks=0, max_seqs_in_block_table=max_seqs, quant_serve=False, num_layers_to_quantize=0,
+               num_layers_to_quantize_max=0)
+    engine = PoolEngine(pool, ecfg, num_layers=L, seg_blocks=0)
+    sched = Scheduler(model, ecfg, num_blocks)
+    engine.scheduler = sched
+    cos_t, sin_t = rotary_tables(D, 4096, device="cuda")
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    max_tok = 8 * 512
+    q = torch.randn((max_tok, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    k = torch.randn((max_tok, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    v = torch.randn((max_tok, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((max_tok, HQ * D), dtype=torch.float16, device=dev)
+
+    n_steps = max(args.steps, 1) * 40
+    # arrivals: gamma(0.5) gaps with a mean of 5 steps per burst of 8 prompts -> ~115 sequences in flight
+    arrival_step, t = [], 0.0
+    while t < n_steps:
+        t += rng.gamma(0.5, 10.0)
+        arrival_step.append(int(t))
+    next_arrival = 0
+    spent = {"schedule": 0.0, "allocate": 0.0, "kernels": 0.0, "free": 0.0}
+    counts = {"prefill_steps": 0, "decode_steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "finished": 0,
+              "allocate_calls": 0, "blocks_allocated": 0, "max_running": 0}
+
+    def dev_i32(x):
+        return torch.tensor(x, dtype=torch.int32, device=dev)
+
+    torch.cuda.synchronize()
+    t_begin = time.perf_counter()
+    for step_no in range(n_steps):
+        while next_arrival < len(arrival_step) and arrival_step[next_arrival] <= step_no:
+            sched.on_requests_arrival([Request(prompt_len=512, max_output_len=int(rng.integers(32, 257)))
+                                       for _ in range(8)])
+            next_arrival += 1
+        t0 = time.perf_counter()
+        batch, swapped_in, swapped_out = sched.get_next_batch(engine)
+        assert not swapped_in and not swapped_out, "the pool is sized so that nothing is evicted"
+        t1 = time.perf_counter()
+        reqs = list(batch)
+        if not reqs:
+            spent["schedule"] += t1 - t0
+            continue
+        prefill = batch is not sched.running_q
+        ids = [r.request_id for r in reqs]
+        lens = [r.prompt_len + r.output_len for r in reqs]
+        new_ids = bm.allocate_blocks_for_seqs(dev_i32(ids), dev_i32(lens))
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if prefill:
+            p_lens, d_lens = [r.prompt_len for r in reqs], []
+            positions = np.concatenate([np.arange(n) for n in p_lens])
+        else:
+            p_lens, d_lens = [], lens
+            positions = np.asarray(lens) - 1
+        n_tok = len(positions)
+        st = build_infer_state(p_lens, ids, d_lens, HKV, D)
+        pos_t = torch.from_numpy(positions).to(dev)
+        st.position_cos, st.position_sin = cos_t[pos_t].contiguous(), sin_t[pos_t].contiguous()
+        for layer in range(L):
+            rotary_embedding_and_store_kvcache(q[:n_tok], k[:n_tok], v[:n_tok], pool.k_cache, pool.v_cache, [], [],
+                                               bm.block_table, model, ecfg, st, layer)
+            if prefill:
+                prefill_attention(q[:n_tok], k[:n_tok], v[:n_tok], o[:n_tok].view(n_tok, HQ, D), model, ecfg, st)
+            else:
+                paged_attention(q[:n_tok], pool.k_cache, pool.v_cache, [], [], bm.block_table, model, ecfg, st,
+                                layer, o[:n_tok])
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        for r in reqs:
+            r.output_len += 1
+        done = [r.request_id for r in reqs if r.is_finished()]
+        if done:
+            bm.free_blocks_for_seqs(dev_i32(done))
+            torch.cuda.synchronize()
+        sched.on_batch_finish(reqs)
+        t4 = time.perf_counter()
+        spent["schedule"] += t1 - t0
+        spent["allocate"] += t2 - t1
+        spent["kernels"] += t3 - t2
+        spent["free"] += t4 - t3
+        counts["prefill_steps" if prefill else "decode_steps"] += 1
+        counts["prefill_tokens" if prefill else "decode_tokens"] += n_tok
+        counts["finished"] += len(done)
+        counts["allocate_calls"] += 1
+        counts["blocks_allocated"] += int(new_ids.numel())
+        counts["max_running"] = max(counts["max_running"], len(sched.running_q))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_begin
+
+    # conservation: every block is free or owned by exactly one running sequence
+    owned = int(bm.num_seq_allocated_blocks.sum().item())
+    free_now = int(bm.is_block_free.sum().item())
+    assert owned + free_now == num_blocks == int(bm.num_free_blocks) + owned, "block accounting drifted"
+    assert owned == sum(-(-(r.prompt_len + r.output_len - 1) // B) for r in sched.running_q), \
+        "running sequences own a different number of blocks than their lengths need"
+    steps_run = counts["prefill_steps"] + counts["decode_steps"]
+    tokens = counts["prefill_tokens"] + counts["decode_tokens"]
+    return {
+        "metric": "KV-path serving loop (scheduler + allocator + rotary/append + attention, 32 layers), 1 MI355X",
+        "value": round(tokens / wall, 1), "unit": "tokens/s (KV path only)", "n_gpus": 1, "steps": steps_run,
+        "warmup": 0, "ms_per_step": round(wall * 1e3 / max(steps_run, 1), 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"cfg4_serving: MHA 32/32, head_dim 128, 32 layers, pool {num_blocks} blocks of 8 MiB, "
+                               "bursts of 8 x 512-token prompts with gamma(0.5) gaps, outputs U[32,256], "
+                               f"{n_steps} scheduler steps, eager launches with a sync per phase for the breakdown"},
+        **counts,
+        "share_of_wall": {kk: round(vv / wall, 4) for kk, vv in spent.items()},
+        "avg_ms": {"schedule": round(spent["schedule"] * 1e3 / n_steps, 4),
+                   "allocate_call": round(spent["allocate"] * 1e3 / max(counts["allocate_calls"], 1), 4),
+                   "kernels_per_step": round(spent["kernels"] * 1e3 / max(steps_run, 1), 4),
+                   "free_and_bookkeeping": round(spent["free"] * 1e3 / max(steps_run, 1), 4)},
+        "roofline": None,
+    }
+
+
 def bench_copy_calibration(args):
     """A plain device copy of known size (the migration kernel moving 512 blocks of
     2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
@@ -787,7 +925,7 @@ def main():
     out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
            "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
            "copy_calibration": bench_copy_calibration, "eviction": bench_eviction,
-           "cfg5_pressure_shrink": bench_pressure_shrink}[args.workload](args)
+           "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}[args.workload](args)
     print(json.dumps(out))
 
 
