@@ -56,7 +56,8 @@ def parse_args():
                          "one-launch-per-layer call)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ctx", type=int, nargs=2, default=[1024, 1536], metavar=("LO", "HI"),
-                    help="decode workloads: context lengths are uniform in [LO, HI] (at most 2048)")
+                    help="decode workloads: context lengths are uniform in [LO, HI]")
+    ap.add_argument("--batch", type=int, default=0, help="decode workloads: number of sequences (0 = the workload's)")
     ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
                     help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
                          "benchmark's definition) or in id order (diagnostic only)")
@@ -91,11 +92,13 @@ def bench_decode(args):
         L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
         default_blocks = 65536
     rng = np.random.default_rng(args.seed)
+    if args.batch:
+        N = args.batch
     lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     num_blocks = args.pool_blocks or default_blocks
-    max_blocks_per_seq = 128
-    max_seqs = 256
+    max_blocks_per_seq = max(128, -(-args.ctx[1] // B))
+    max_seqs = max(256, N)
 
     # block tables: a seeded permutation of the whole pool dealt in order
     perm = rng.permutation(num_blocks)
@@ -389,7 +392,7 @@ def bench_resize(args):
 
 
 def bench_pressure_shrink(args):
-    """Config 5 as BASELINE states it: CodeLlama-34B-shaped decode on a ~200 GB pool, and
+    """Config 5 with its mid-run shrink: CodeLlama-34B-shaped decode on a ~200 GB pool, and
     mid-run the scheduler's own give-back rule releases 25 % of the blocks (63 578 -> 47 684)
     while a quarter of the live blocks sit above the cut and have to move."""
     import torch
