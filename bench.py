@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # FETCH_SIZE and WRITE_SIZE counters scaled by a device copy of known size
 # (profiles/attn_decode_phase1_mfma_cfg2_pmc_traffic.md); counters cannot be
 # collected from inside this process.
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 343_659_871
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 343_622_787
 
 
 class Cfg:
