@@ -7,7 +7,7 @@ import torch
 
 from oracle import ref_cpu as R
 from helpers import make_case
-from gpu_helpers import assert_state_equal, bits, load_manager, manager_state
+from gpu_helpers import pool_bytes, pool_case, assert_state_equal, bits, load_manager, manager_state
 from morphserve_amd import BlockManager, ElasticKVPool, swiftllm_c
 from morphserve_amd.worker.kernels import block_mgmt
 
@@ -136,58 +136,10 @@ def test_carve_segment_and_acquire(cuda):
     assert float(k[1, 0, 1, 2, 3]) == 5.0
 
 
-def _pool_case(cuda, seed, org, S, nseg, live_frac, L=2, Hkv=2, D=128):
-    """ElasticKVPool grown to org + nseg*S blocks with a random live set, plus the
-    oracle's mirror of it (arena + layout with an explicit segment table)."""
-    rng = np.random.default_rng(seed)
-    total = org + nseg * S
-    pool = ElasticKVPool(org, L, Hkv, 16, D, max_seqs_in_block_table=24, max_blocks_per_seq=total)
-    for _ in range(nseg):
-        pool.expand(S)
-    blk = L * Hkv * 16 * D
-    # oracle arena: base K, base V, then per segment K, V
-    lay = R.PoolLayout(L, Hkv, 16, D, k_base=0, v_base=org * blk, num_blocks_org=org, seg_blocks=S,
-                       k_seg=[2 * org * blk + j * 2 * S * blk for j in range(nseg)],
-                       v_seg=[2 * org * blk + j * 2 * S * blk + S * blk for j in range(nseg)])
-    arena = rng.standard_normal(2 * total * blk, dtype=np.float32).astype(np.float16)
-    pool.k_cache.copy_(torch.from_numpy(arena[:org * blk]).view_as(pool.k_cache))
-    pool.v_cache.copy_(torch.from_numpy(arena[org * blk:2 * org * blk]).view_as(pool.v_cache))
-    for j in range(nseg):
-        pool.k_cache_new[j].copy_(torch.from_numpy(arena[lay.k_seg[j]:lay.k_seg[j] + S * blk]).view_as(pool.k_cache_new[j]))
-        pool.v_cache_new[j].copy_(torch.from_numpy(arena[lay.v_seg[j]:lay.v_seg[j] + S * blk]).view_as(pool.v_cache_new[j]))
-    # random live set scattered over the whole range, dealt to sequences
-    n_live = int(live_frac * total)
-    live = np.random.default_rng(seed + 1000).permutation(total)[:n_live]
-    ob = R.BlockManagerOracle("GPU", org, 24, total, 16)
-    for _ in range(nseg):
-        ob.expand(S)
-    cuts = np.sort(rng.choice(np.arange(1, n_live), size=min(11, n_live - 1), replace=False))
-    for s, ids in enumerate(np.split(live, cuts)):
-        ob.block_table[s, :len(ids)] = ids
-        ob.num_seq_allocated_blocks[s] = len(ids)
-    ob.is_block_free[live] = False
-    ob.num_free_blocks = total - n_live
-    # a freed row with stale ids that must stay untouched
-    ob.block_table[20, :3] = [total - 1, 0, total - 2]
-    bm = pool.block_manager
-    bm.block_table.copy_(torch.from_numpy(ob.block_table))
-    bm.num_seq_allocated_blocks.copy_(torch.from_numpy(ob.num_seq_allocated_blocks))
-    bm.is_block_free.copy_(torch.from_numpy(ob.is_block_free))
-    bm.num_free_blocks = ob.num_free_blocks
-    return pool, ob, arena, lay
-
-
-def _pool_bytes(pool):
-    parts = [pool.k_cache.reshape(-1), pool.v_cache.reshape(-1)]
-    for k, v in zip(pool.k_cache_new, pool.v_cache_new):
-        parts += [k.reshape(-1), v.reshape(-1)]
-    return bits(torch.cat(parts))
-
-
 @pytest.mark.parametrize("seed,org,S,nseg,keep,live_frac", [(0, 16, 8, 4, 1, 0.3), (1, 32, 16, 6, 2, 0.45),
                                                            (2, 8, 4, 5, 0, 0.15)])
 def test_shrink_with_migration_bit_exact(cuda, seed, org, S, nseg, keep, live_frac):
-    pool, ob, arena, lay = _pool_case(cuda, seed, org, S, nseg, live_frac)
+    pool, ob, arena, lay = pool_case(cuda, seed, org, S, nseg, live_frac)
     new_n = org + keep * S
     want_src, want_dst = R.apply_migration(arena, lay, ob, new_n)
     src, dst = pool.shrink_to(new_n)
@@ -197,17 +149,17 @@ def test_shrink_with_migration_bit_exact(cuda, seed, org, S, nseg, keep, live_fr
     assert len(pool.k_cache_new) == keep and pool.num_blocks == new_n
     blk = lay.block_elems
     kept = 2 * org * blk + keep * 2 * S * blk
-    assert np.array_equal(_pool_bytes(pool), arena[:kept].view(np.uint16))
+    assert np.array_equal(pool_bytes(pool), arena[:kept].view(np.uint16))
 
 
 def test_shrink_refused_when_live_blocks_do_not_fit(cuda):
-    pool, ob, arena, lay = _pool_case(cuda, 3, 8, 8, 3, 0.6)
+    pool, ob, arena, lay = pool_case(cuda, 3, 8, 8, 3, 0.6)
     before_state = manager_state(pool.block_manager)
-    before_bytes = _pool_bytes(pool).copy()
+    before_bytes = pool_bytes(pool).copy()
     with pytest.raises(RuntimeError, match="cannot shrink"):
         pool.shrink_to(8)
     assert_state_equal(manager_state(pool.block_manager), before_state, "refused shrink")
-    assert np.array_equal(_pool_bytes(pool), before_bytes)
+    assert np.array_equal(pool_bytes(pool), before_bytes)
     assert len(pool.k_cache_new) == 3
 
 

@@ -6,9 +6,8 @@ import pytest
 import torch
 
 from oracle import ref_cpu as R
-from gpu_helpers import assert_state_equal, bits, manager_state
+from gpu_helpers import assert_state_equal, bits, manager_state, pool_bytes, pool_case
 from morphserve_amd import KVSwapper, _capi
-from test_gpu_block_manager import _pool_bytes, _pool_case
 
 pytestmark = pytest.mark.gpu
 
@@ -24,7 +23,7 @@ def _oracle_swap(arena, lay, src_bm, dst_bm, ks, vs, seq_ids, is_swap_in):
 @pytest.mark.parametrize("use_kernel,pinned", [(True, True), (False, True), (False, False)])
 def test_swap_out_and_back_matches_the_oracle(cuda, use_kernel, pinned):
     org, S, nseg = 16, 8, 3
-    pool, ob, arena, lay = _pool_case(cuda, 5, org, S, nseg, 0.5)
+    pool, ob, arena, lay = pool_case(cuda, 5, org, S, nseg, 0.5)
     n_cpu = 40
     sw = KVSwapper(pool, n_cpu, pinned=pinned)
     assert sw.k_swap.is_pinned() == pinned
@@ -40,7 +39,7 @@ def test_swap_out_and_back_matches_the_oracle(cuda, use_kernel, pinned):
         assert_state_equal(manager_state(sw.gpu_block_manager), ob.snapshot(), what + " gpu manager")
         assert_state_equal(manager_state(sw.cpu_block_manager), ocpu.snapshot(), what + " cpu manager")
         assert np.array_equal(bits(sw.k_swap), bits(ks)) and np.array_equal(bits(sw.v_swap), bits(vs)), what
-        assert np.array_equal(_pool_bytes(pool), arena[:full].view(np.uint16)), what
+        assert np.array_equal(pool_bytes(pool), arena[:full].view(np.uint16)), what
 
     n = sw.swap_out_seqs(out1, use_kernel=use_kernel)
     assert n == _oracle_swap(arena, lay, ob, ocpu, ks, vs, out1, False) > 0
@@ -69,7 +68,7 @@ def test_swap_out_and_back_matches_the_oracle(cuda, use_kernel, pinned):
 
 def test_device_id_route_rejects_pageable_swap_space(cuda):
     import ctypes as C
-    pool, ob, arena, lay = _pool_case(cuda, 6, 8, 4, 1, 0.3)
+    pool, ob, arena, lay = pool_case(cuda, 6, 8, 4, 1, 0.3)
     sw = KVSwapper(pool, 8, pinned=False)
     rows = [s for s in range(24) if ob.num_seq_allocated_blocks[s] > 0][:1]
     before = manager_state(sw.gpu_block_manager)
