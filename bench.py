@@ -673,7 +673,7 @@ def bench_serving(args):
     Every step runs scheduler -> block allocation -> rotary + append -> attention for all 32
     layers -> frees.  Reports where the time of a step goes."""
     import torch
-    from morphserve_amd import (ElasticKVPool, build_infer_state, paged_attention, prefill_attention,
+    from morphserve_amd import (ElasticKVPool, build_infer_state, decode_rope_append_and_attend, prefill_attention,
                                 rotary_embedding_and_store_kvcache, rotary_tables)
     from morphserve_amd.server import PoolEngine, Request, Scheduler
 
@@ -748,13 +748,13 @@ def bench_serving(args):
         pos_t = torch.from_numpy(positions).to(dev)
         st.position_cos, st.position_sin = cos_t[pos_t].contiguous(), sin_t[pos_t].contiguous()
         for layer in range(L):
-            rotary_embedding_and_store_kvcache(q[:n_tok], k[:n_tok], v[:n_tok], pool.k_cache, pool.v_cache, [], [],
-                                               bm.block_table, model, ecfg, st, layer)
-            if prefill:
+            if prefill:       # rotary + append in one launch, then causal attention over the batch's own k, v
+                rotary_embedding_and_store_kvcache(q[:n_tok], k[:n_tok], v[:n_tok], pool.k_cache, pool.v_cache,
+                                                   [], [], bm.block_table, model, ecfg, st, layer)
                 prefill_attention(q[:n_tok], k[:n_tok], v[:n_tok], o[:n_tok].view(n_tok, HQ, D), model, ecfg, st)
-            else:
-                paged_attention(q[:n_tok], pool.k_cache, pool.v_cache, [], [], bm.block_table, model, ecfg, st,
-                                layer, o[:n_tok])
+            else:             # rotary + append + attention in one launch
+                decode_rope_append_and_attend(k[:n_tok], v[:n_tok], q[:n_tok], pool.k_cache, pool.v_cache, [], [],
+                                              bm.block_table, model, ecfg, st, layer, o[:n_tok])
         torch.cuda.synchronize()
         t3 = time.perf_counter()
         for r in reqs:

@@ -120,6 +120,21 @@ int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,
                            float softmax_scale, int32_t layer, int32_t tokens_per_split,
                            int32_t max_splits, void* mid_o, void* mid_lse, void* stream);
 
+/* rotary_embedding_inplace (decode rows) + store_kvcache + paged_attention of one
+ * layer in ONE launch: MS/worker/layers/transformer_layer.py:93-126, :181-187
+ * for a decode batch.  q and k arrive UNROTATED; row i of cos_table / sin_table
+ * ([n, D/2] fp16) belongs to sequence i's new token.  q and the new k row are
+ * rotated on their way in (arithmetic of mkv_rope_store_kvcache), the rotated k
+ * row and the v row are written to the cache, attention uses both.  Unlike the
+ * separate rotary call, q and k themselves are left as they were. */
+int mkv_decode_rope_append_attn(const void* k, const void* v, const void* q,
+                                const void* cos_table, const void* sin_table, void* o,
+                                const mkv_pool* pool, const int32_t* block_table,
+                                int64_t max_blocks_per_seq, const int32_t* seq_ids,
+                                const int32_t* seq_lens, int32_t n, int32_t num_q_heads,
+                                float softmax_scale, int32_t layer, int32_t tokens_per_split,
+                                int32_t max_splits, void* mid_o, void* mid_lse, void* stream);
+
 /* Tuning knob without a counterpart in the reference: which phase-1 kernel
  * mkv_paged_attn_decode launches.  0 = by GQA group size (matrix cores when
  * Hq/Hkv >= 4, vector ALU otherwise), 1 = vector ALU, 2 = matrix cores. */

@@ -22,7 +22,8 @@ from . import _capi  # noqa: F401
 from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
 from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
-from .worker.kernels.paged_attn import decode_append_and_attend, paged_attention  # noqa: F401
+from .worker.kernels.paged_attn import (decode_append_and_attend, decode_rope_append_and_attend,  # noqa: F401
+                                        paged_attention)
 from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401
 from .worker.kernels.rotary_emb import (rotary_embedding_and_store_kvcache, rotary_embedding_inplace,  # noqa: F401
                                         rotary_tables)

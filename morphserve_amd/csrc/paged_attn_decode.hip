@@ -10,6 +10,7 @@
 // online-softmax state (fp32, base 2), merged across rows and waves at the end.
 // Phase 2 merges the per-split partials by log-sum-exp.
 #include "common.h"
+#include "rope_math.h"
 
 namespace mkv {
 
@@ -149,7 +150,9 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const int32_t* __restrict__ seq_ids, const int32_t* __restrict__ seq_lens, float scale2,
     int32_t layer, int32_t blocks_per_split, int32_t max_splits,
     const uint4* __restrict__ k_new,    // [n, Hkv, D] fp16 or NULL: token len-1 to append first
-    const uint4* __restrict__ v_new) {
+    const uint4* __restrict__ v_new,
+    const uint4* __restrict__ cos_t,    // [n, D/2] fp16 or NULL: rotate q and the new k row on the way in
+    const uint4* __restrict__ sin_t) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -178,6 +181,18 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
 #pragma unroll
     for (int g = 0; g < G; ++g)
         qreg[g] = q[((int64_t)i * Hq + kvh * G + g) * (kD / 8) + (lane & 15)];
+    // rotary on the way in: chunk c pairs with chunk c ^ 8 (dims d and d + 64)
+    const bool rope = cos_t != nullptr;
+    uint4 cosc = make_uint4(0u, 0u, 0u, 0u), sinc = cosc;
+    if (rope) {
+        cosc = cos_t[(int64_t)i * (kD / 16) + (lane & 7)];
+        sinc = sin_t[(int64_t)i * (kD / 16) + (lane & 7)];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const uint4 partner = q[((int64_t)i * Hq + kvh * G + g) * (kD / 8) + ((lane & 15) ^ 8)];
+            qreg[g] = rotate_own_half(qreg[g], partner, cosc, sinc, (lane & 8) != 0);
+        }
+    }
 
     RowState<G> st;
 #pragma unroll
@@ -261,8 +276,12 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
                     // token len-1: write it into its slot of the cache and use it from
                     // registers, whatever the slot held before
                     const int off = (len - 1) & (kB - 1);
-                    const uint4 kn = k_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + (lane & 15)];
+                    uint4 kn = k_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + (lane & 15)];
                     const uint4 vn = v_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + (lane & 15)];
+                    if (rope) {
+                        const uint4 partner = k_new[((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + ((lane & 15) ^ 8)];
+                        kn = rotate_own_half(kn, partner, cosc, sinc, (lane & 8) != 0);
+                    }
                     if (r == (off & 3)) {
                         BlockAddr a = block_addr(pool, pid, block_bytes);
                         const int64_t slot = head_off + (int64_t)off * (kD * 2) + (lane & 15) * 16;
@@ -356,7 +375,8 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     float* __restrict__ mid_lse, const mkv_pool pool, const int32_t* __restrict__ block_table,
     int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ seq_lens, float scale2, int32_t layer, int32_t blocks_per_split,
-    int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new) {
+    int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new,
+    const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t) {
     __shared__ __attribute__((aligned(16))) char stage[4][2][kLdsTile];
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
@@ -389,6 +409,14 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         const uint4* qp = q + ((int64_t)i * Hq + kvh * G + n) * (kD / 8) + c * 4;
 #pragma unroll
         for (int x = 0; x < 4; ++x) qb[x] = __builtin_bit_cast(v8h, qp[x]);
+        if (cos_t != nullptr) {       // rotary on the way in: dims c*32.. pair with dims (c^2)*32..
+            const uint4* pp = q + ((int64_t)i * Hq + kvh * G + n) * (kD / 8) + (c ^ 2) * 4;
+            const uint4* cp = cos_t + (int64_t)i * (kD / 16) + (c & 1) * 4;
+            const uint4* sp = sin_t + (int64_t)i * (kD / 16) + (c & 1) * 4;
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                qb[x] = __builtin_bit_cast(v8h, rotate_own_half(__builtin_bit_cast(uint4, qb[x]), pp[x], cp[x], sp[x], c >= 2));
+        }
     } else {
 #pragma unroll
         for (int x = 0; x < 4; ++x) qb[x] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
@@ -448,7 +476,13 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         if (lane < 32) {
             const bool is_v = lane >= 16;
             const int64_t src = ((int64_t)i * pool.num_kv_heads + kvh) * (kD / 8) + n;
-            const v4u val = __builtin_bit_cast(v4u, is_v ? v_new[src] : k_new[src]);
+            v4u val = __builtin_bit_cast(v4u, is_v ? v_new[src] : k_new[src]);
+            if (cos_t != nullptr && !is_v) {    // the new k row is rotated before it is stored and used
+                const uint4 partner = k_new[src - n + (n ^ 8)];
+                const uint4 cc = cos_t[(int64_t)i * (kD / 16) + (n & 7)];
+                const uint4 ss = sin_t[(int64_t)i * (kD / 16) + (n & 7)];
+                val = __builtin_bit_cast(v4u, rotate_own_half(__builtin_bit_cast(uint4, val), partner, cc, ss, n >= 8));
+            }
             BlockAddr a = block_addr(pool, pid, block_bytes);
             const int64_t slot = head_off + (int64_t)off * (kD * 2) + n * 16;
             *(v4u*)(const_cast<char*>(is_v ? a.v : a.k) + slot) = val;
@@ -591,18 +625,19 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
                           int64_t max_blocks_per_seq, const int32_t* seq_ids,
                           const int32_t* seq_lens, float scale2, int32_t layer,
                           int32_t blocks_per_split, int32_t max_splits, const void* k_new,
-                          const void* v_new) {
+                          const void* v_new, const void* cos_t, const void* sin_t) {
     const bool mfma = g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
     if (mfma) {
         hipLaunchKernelGGL(attn_decode_phase1_mfma<G>, grid, dim3(256), 0, s, (const uint4*)q,
                            (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
                            max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
-                           max_splits, (const uint4*)k_new, (const uint4*)v_new);
+                           max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
+                           (const uint4*)sin_t);
     } else {
         hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
                            (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
                            seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
-                           (const uint4*)k_new, (const uint4*)v_new);
+                           (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t);
     }
 }
 
@@ -630,7 +665,8 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
                        int64_t max_blocks_per_seq, const int32_t* seq_ids, const int32_t* seq_lens,
                        int32_t n, int32_t num_q_heads, float softmax_scale, int32_t layer,
                        int32_t tokens_per_split, int32_t max_splits, void* mid_o, void* mid_lse,
-                       const void* k_new, const void* v_new, void* stream) {
+                       const void* k_new, const void* v_new, const void* cos_t, const void* sin_t,
+                       void* stream) {
     int rc = mkv::check_pool(pool);
     if (rc) return rc;
     MKV_REQUIRE(n >= 0, "n must be >= 0");
@@ -659,7 +695,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
     case GG:                                                                                       \
         mkv::launch_phase1<GG>(grid, s, q, o, mid_o, mid_lse, pool, block_table,                   \
                                max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, bps,          \
-                               max_splits, k_new, v_new);                                          \
+                               max_splits, k_new, v_new, cos_t, sin_t);                            \
         break;
             MKV_CASE(1)
             MKV_CASE(2)
@@ -690,7 +726,7 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
                           void* mid_lse, void* stream) {
     return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
                        num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
-                       mid_lse, nullptr, nullptr, stream);
+                       mid_lse, nullptr, nullptr, nullptr, nullptr, stream);
 }
 
 int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,
@@ -703,7 +739,23 @@ int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,
     MKV_REQUIRE(((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0, "k/v must be 16-byte aligned");
     return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
                        num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
-                       mid_lse, k, v, stream);
+                       mid_lse, k, v, nullptr, nullptr, stream);
+}
+
+int mkv_decode_rope_append_attn(const void* k, const void* v, const void* q, const void* cos_table,
+                                const void* sin_table, void* o, const mkv_pool* pool,
+                                const int32_t* block_table, int64_t max_blocks_per_seq,
+                                const int32_t* seq_ids, const int32_t* seq_lens, int32_t n,
+                                int32_t num_q_heads, float softmax_scale, int32_t layer,
+                                int32_t tokens_per_split, int32_t max_splits, void* mid_o, void* mid_lse,
+                                void* stream) {
+    MKV_REQUIRE(n == 0 || (k && v && cos_table && sin_table), "k/v/cos/sin are NULL");
+    MKV_REQUIRE(((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0 && ((uintptr_t)cos_table & 15) == 0 &&
+                    ((uintptr_t)sin_table & 15) == 0,
+                "k/v/cos/sin must be 16-byte aligned");
+    return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
+                       num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
+                       mid_lse, k, v, cos_table, sin_table, stream);
 }
 
 }  // extern "C"

@@ -9,10 +9,9 @@
 //     out[d + D/2]  = fma(x[d], sin[d],   x[d + D/2] * cos[d])        d < D/2
 // (the contraction a compiler applies to "a*b - c*d" / "a*b + c*d" with fp16 operands).
 #include "common.h"
+#include "rope_math.h"
 
 namespace mkv {
-
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 
 struct RopeArgs {
     __half* q;                    // [T, Hq, D], rotated in place
@@ -34,17 +33,6 @@ struct RopeArgs {
     int32_t head_dim;
     int32_t layer;
 };
-
-__device__ __forceinline__ void rotate8(const h8 x0, const h8 x1, const h8 c, const h8 s, h8& o0, h8& o1) {
-#pragma clang fp contract(off)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const _Float16 p0 = x1[e] * s[e];          // rounded to fp16 on its own
-        const _Float16 p1 = x1[e] * c[e];
-        o0[e] = __builtin_fmaf16(x0[e], c[e], -p0);
-        o1[e] = __builtin_fmaf16(x0[e], s[e], p1);
-    }
-}
 
 // One workgroup per token.  Units of eight rotation pairs: q heads first, then k heads,
 // then (STORE) the 16-byte units of the v row.

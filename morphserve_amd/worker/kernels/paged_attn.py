@@ -105,6 +105,48 @@ def decode_append_and_attend(
         cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
 
 
+def decode_rope_append_and_attend(
+    k: torch.Tensor,                    # [num_decoding_seqs, num_kv_heads, head_dim], NOT yet rotated
+    v: torch.Tensor,
+    q: torch.Tensor,                    # [num_decoding_seqs, num_q_heads, head_dim], NOT yet rotated
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_cache_new: List[torch.Tensor],
+    v_cache_new: List[torch.Tensor],
+    block_table: torch.Tensor,
+    model_config,
+    engine_config,
+    infer_state,                        # with position_cos / position_sin, one row per decoding sequence
+    cur_layer: int,
+    o: torch.Tensor,
+) -> None:
+    """``rotary_embedding_inplace`` + ``store_kvcache`` + ``paged_attention`` of a decode-only
+    batch (MorphServe/worker/layers/transformer_layer.py:93-126, :181-187) as ONE launch per
+    layer.  q and k are rotated on their way into the kernel and are left unrotated in
+    memory; the cache receives the rotated k row."""
+    assert infer_state.num_prefill_seqs == 0, "the fused call covers decode-only batches"
+    assert k.is_contiguous() and v.is_contiguous() and q.is_contiguous() and o.is_contiguous()
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and block_table.is_contiguous()
+    assert q.dtype == torch.float16 and o.dtype == torch.float16 and k.dtype == torch.float16
+    cos, sin = infer_state.position_cos, infer_state.position_sin
+    n = infer_state.num_decoding_seqs
+    if n == 0:
+        return
+    hq, d = model_config.num_q_heads, model_config.head_dim
+    assert cos is not None and sin is not None and cos.is_contiguous() and sin.is_contiguous()
+    assert cos.dtype == torch.float16 and tuple(cos.shape) == (n, d // 2) == tuple(sin.shape)
+    tps, splits = _split_for(infer_state, model_config, engine_config)
+    pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
+    mid_o, mid_lse = (None, None)
+    if splits > 1:
+        mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
+    _capi.check(_capi.lib().mkv_decode_rope_append_attn(
+        k.data_ptr(), v.data_ptr(), q.data_ptr(), cos.data_ptr(), sin.data_ptr(), o.data_ptr(), C.byref(pool),
+        block_table.data_ptr(), block_table.shape[1], infer_state.seq_ids.data_ptr(),
+        infer_state.decoding_seq_lens.data_ptr(), n, hq, float(infer_state.softmax_scale),
+        cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
+
+
 def paged_attention(
     q: torch.Tensor,                    # [num_decoding_seqs, num_q_heads, head_dim]
     k_cache: torch.Tensor,              # [num_blocks, num_layers, num_kv_heads, block_size, head_dim]

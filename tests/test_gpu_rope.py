@@ -82,3 +82,47 @@ def test_fused_rotary_store_equals_rotate_then_append(cuda, seed, L, Hq, Hkv, la
     kc2, vc2, _ = to_gpu(make_case(seed, L, Hq, Hkv, lens, num_blocks=nblk, fill="all"), cuda)
     store_kvcache(kg, vg, kc2, vc2, [], [], bt, model, engine, state, layer)
     assert np.array_equal(bits(kc2), bits(kc)) and np.array_equal(bits(vc2), bits(vc))
+
+
+@pytest.mark.parametrize("Hq,Hkv,variant", [(32, 32, 1), (8, 4, 1), (32, 8, 2), (64, 8, 2)])
+@pytest.mark.parametrize("target_wgs", [1, 100000])
+def test_decode_with_rotary_append_and_attention_in_one_launch(cuda, Hq, Hkv, variant, target_wgs):
+    """q and k go in unrotated: the cache must receive exactly the rotated k row (and v), the
+    output must be the attention of the rotated q over the updated cache, q and k stay as given."""
+    from helpers import assert_attn_close
+    from morphserve_amd import _capi, decode_rope_append_and_attend
+    from morphserve_amd.worker.kernels import paged_attn as PA
+    lens = [1, 16, 17, 200, 1024, 1535, 64]
+    nblk = sum((x + 15) // 16 for x in lens) + 4
+    layer, L = 1, 2
+    case = make_case(7, L, Hq, Hkv, lens, num_blocks=nblk, fill="live")
+    kc, vc, bt = to_gpu(case, cuda)
+    rng = np.random.default_rng(70)
+    n = len(lens)
+    q, k, v = rand_f16(rng, n, Hq, case.D), rand_f16(rng, n, Hkv, case.D), rand_f16(rng, n, Hkv, case.D)
+    ct, st_ = RO.rotary_tables(case.D, 2048)
+    pos = np.asarray(lens) - 1
+    cos, sin = np.ascontiguousarray(ct[pos]), np.ascontiguousarray(st_[pos])
+    model, engine = configs(case)
+    state = build_infer_state([], case.seq_ids.tolist(), lens, Hkv, case.D)
+    state.position_cos = torch.from_numpy(cos).to(cuda)
+    state.position_sin = torch.from_numpy(sin).to(cuda)
+    qg, kg, vg = (torch.from_numpy(x).to(cuda) for x in (q, k, v))
+    o = torch.full((n, Hq * case.D), float("nan"), dtype=torch.float16, device=cuda)
+    old = PA.TARGET_WORKGROUPS
+    PA.TARGET_WORKGROUPS = target_wgs
+    _capi.check(_capi.lib().mkv_set_decode_variant(variant))
+    try:
+        decode_rope_append_and_attend(kg, vg, qg, kc, vc, [], [], bt, model, engine, state, layer, o)
+        torch.cuda.synchronize()
+    finally:
+        PA.TARGET_WORKGROUPS = old
+        _capi.lib().mkv_set_decode_variant(0)
+    assert np.array_equal(bits(qg), bits(q)) and np.array_equal(bits(kg), bits(k))      # inputs untouched
+    q_rot, k_rot = q.copy(), k.copy()
+    RO.rotary_embedding_inplace(q_rot, k_rot, cos, sin)
+    R.append_decode(case.arena, case.lay, k_rot, v, case.block_table, case.seq_ids, np.asarray(lens), layer)
+    assert np.array_equal(bits(kc), bits(case.k_pool)) and np.array_equal(bits(vc), bits(case.v_pool))
+    want = R.paged_attention(q_rot, case.arena, case.lay, case.block_table, case.seq_ids, np.asarray(lens),
+                             case.D ** -0.5, layer)
+    assert_attn_close(o.cpu().numpy().reshape(n, Hq, case.D), np.asarray(want), "rotary + append + attention")
