@@ -60,7 +60,7 @@ def update_kvcache_after_replacing_layer(engine: PoolEngine, layer_id: int) -> N
         model.pool.expand(model.kv_cache_new_block_size)
     else:
         model.pool.expand(int(seg[0].shape[0]), seg[0], seg[1])
-    model.kv_cache_new_block_size = model.pool.kv_cache_new_block_size
+        model.kv_cache_new_block_size = int(seg[0].shape[0])
     if engine.scheduler is not None:
         engine.scheduler.num_gpu_blocks += model.kv_cache_new_block_size
 
@@ -91,7 +91,10 @@ def quant2org_and_update_kvcache(engine: PoolEngine, update_kvcache: bool = True
         raise RuntimeError("no replaced layer to restore")
     if update_kvcache:
         pool = model.pool
-        if pool.shrink_tail_if_unused():
+        contiguous = hasattr(pool, "tail_unused")          # a virtual-memory pool: no segments to pop
+        if contiguous and pool.tail_unused(model.kv_cache_new_block_size):
+            pool.shrink_to(pool.num_blocks - model.kv_cache_new_block_size)
+        elif not contiguous and pool.shrink_tail_if_unused():
             pass
         elif not engine.migrate:
             return False

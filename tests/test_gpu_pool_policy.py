@@ -9,7 +9,7 @@ import torch
 from oracle import ref_cpu as R
 from helpers import Cfg, rand_f16
 from gpu_helpers import assert_state_equal, bits, manager_state
-from morphserve_amd import ElasticKVPool, build_infer_state, store_kvcache
+from morphserve_amd import ElasticKVPool, VmmKVPool, build_infer_state, store_kvcache
 from morphserve_amd.server import (PoolEngine, Request, Scheduler, org2quant_and_update_kvcache,
                                    quant2org_and_update_kvcache)
 
@@ -22,8 +22,15 @@ ORG, S, MAX_SEG = 16, 8, 4
 class Mirror:
     """Oracle-side twin of the pool: arena with room for MAX_SEG segments + block manager."""
 
-    def __init__(self):
+    def __init__(self, contiguous=False):
         blk = L * HKV * B * D
+        self.contiguous = contiguous
+        if contiguous:                       # one K tensor and one V tensor with room for every segment
+            self.lay = R.plain_layout(ORG + MAX_SEG * S, L, HKV, B, D)
+            self.arena = np.zeros(2 * (ORG + MAX_SEG * S) * blk, dtype=np.float16)
+            self.bm = R.BlockManagerOracle("GPU", ORG, 16, 32, B)
+            self.nseg = 0
+            return
         self.lay = R.PoolLayout(L, HKV, B, D, k_base=0, v_base=ORG * blk, num_blocks_org=ORG, seg_blocks=S,
                                 k_seg=[2 * ORG * blk + j * 2 * S * blk for j in range(MAX_SEG)],
                                 v_seg=[2 * ORG * blk + j * 2 * S * blk + S * blk for j in range(MAX_SEG)])
@@ -39,15 +46,21 @@ def _pool_bytes(pool):
     return bits(torch.cat(parts))
 
 
-def test_pressure_driven_growth_and_migrating_give_back(cuda):
+@pytest.mark.parametrize("backing", ["segments", "virtual_memory"])
+def test_pressure_driven_growth_and_migrating_give_back(cuda, backing):
     rng = np.random.default_rng(11)
+    vmm = backing == "virtual_memory"
     ecfg = Cfg(block_size=B, max_batch_size=8, max_tokens_in_batch=4096, num_cpu_blocks=64,
                max_seqs_in_block_table=16, max_blocks_per_seq=32, quant_serve=True,
                num_layers_to_quantize=2, num_layers_to_quantize_max=0)
     mcfg = Cfg(num_layers=L, num_q_heads=HKV, num_kv_heads=HKV, head_dim=D)
-    pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=16, max_blocks_per_seq=32)
+    if vmm:
+        pool = VmmKVPool(ORG, ORG + MAX_SEG * S, L, HKV, B, D, max_seqs_in_block_table=16, max_blocks_per_seq=32,
+                         chunk_blocks=S)
+    else:
+        pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=16, max_blocks_per_seq=32)
     engine = PoolEngine(pool, ecfg, num_layers=6, seg_blocks=S, migrate=True)
-    mir = Mirror()
+    mir = Mirror(contiguous=vmm)
     events = []
 
     def grow(e):
@@ -141,6 +154,7 @@ def test_pressure_driven_growth_and_migrating_give_back(cuda):
     step()   # 17 free >= 2 segments' worth, nothing waiting: both segments go, live blocks move below 16
     assert events == ["grow", "grow", "migrate4", "migrate8"], events
     assert pool.num_blocks == 16 and sched.num_gpu_blocks == 16 and len(pool.k_cache_new) == 0
+    assert tuple(pool.k_cache.shape)[0] == 16
     assert engine.model.next_unquantized_layer == 5 and engine.model.layer_quant_list == []
     for _ in range(3):
         step()                                              # appends keep landing through the rewritten tables
@@ -151,8 +165,14 @@ def test_pressure_driven_growth_and_migrating_give_back(cuda):
     step()
 
     # every byte of the pool, and the logical KV of each live sequence through its table
-    keep = 2 * ORG * mir.lay.block_elems + len(pool.k_cache_new) * 2 * S * mir.lay.block_elems
-    assert np.array_equal(_pool_bytes(pool), mir.arena[:keep].view(np.uint16))
+    if vmm:
+        nb, cap, be = pool.num_blocks, ORG + MAX_SEG * S, mir.lay.block_elems
+        assert pool.k_cache_new == [] and nb in (16, 32)
+        assert np.array_equal(bits(pool.k_cache).reshape(-1), mir.arena[:nb * be].view(np.uint16))
+        assert np.array_equal(bits(pool.v_cache).reshape(-1), mir.arena[cap * be:(cap + nb) * be].view(np.uint16))
+    else:
+        keep = 2 * ORG * mir.lay.block_elems + len(pool.k_cache_new) * 2 * S * mir.lay.block_elems
+        assert np.array_equal(_pool_bytes(pool), mir.arena[:keep].view(np.uint16))
     table = bm.block_table.cpu().numpy()
     caches = {"k": [pool.k_cache] + pool.k_cache_new, "v": [pool.v_cache] + pool.v_cache_new}
     for r in sched.running_q:
@@ -164,8 +184,10 @@ def test_pressure_driven_growth_and_migrating_give_back(cuda):
                 rows = []
                 for j in range((n + B - 1) // B):
                     pid = int(table[r.request_id, j])
-                    seg, local = (0, pid) if pid < ORG else (1 + (pid - ORG) // S, (pid - ORG) % S)
+                    seg, local = (0, pid) if (vmm or pid < ORG) else (1 + (pid - ORG) // S, (pid - ORG) % S)
                     blkt = caches[which][seg][local, layer].cpu().numpy()        # [Hkv, B, D]
                     rows.append(np.transpose(blkt, (1, 0, 2)))
                 got = np.concatenate(rows, axis=0)[:n]
                 assert np.array_equal(bits(got), bits(want)), (r.request_id, layer, which)
+    if vmm:
+        pool.close()

@@ -148,3 +148,43 @@ def test_append_and_attention_on_mapped_memory(cuda):
         assert_attn_close(o.cpu().numpy().reshape(len(lens), 2 * HKV, D), np.asarray(want_o), "attention on the grown pool")
     finally:
         pool.close()
+
+
+def test_eviction_on_a_virtual_memory_pool(cuda):
+    """KVSwapper over a grown VmmKVPool: ids beyond the first size are swapped like any other."""
+    from morphserve_amd import KVSwapper
+    pool = VmmKVPool(16, 64, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=32, chunk_blocks=16)
+    try:
+        pool.expand(16)
+        rng = np.random.default_rng(9)
+        arena = _mirror(pool, 32, rng)
+        lay = R.plain_layout(32, L, HKV, B, D)
+        bm = pool.block_manager
+        ob = R.BlockManagerOracle("GPU", 32, 8, 32, B)
+        ids, lens = [2, 5, 0], [16 * 9, 16 * 12, 40]
+        bm.allocate_blocks_for_seqs(_i32(ids, cuda), _i32(lens, cuda))
+        ob.allocate_blocks_for_seqs(ids, lens)
+        sw = KVSwapper(pool, 24)
+        ocpu = R.BlockManagerOracle("CPU", 24, 8, 32, B)
+        ks, vs = np.zeros(sw.k_swap.shape, np.float16), np.zeros(sw.v_swap.shape, np.float16)
+
+        def oracle_swap(src_bm, dst_bm, seqs, is_in):
+            ln = src_bm.get_num_allocated_blocks(seqs) * B
+            src = src_bm.gather_allocated_blocks_and_free(seqs)
+            dst = dst_bm.allocate_blocks_for_seqs(seqs, ln)
+            R.swap_blocks(arena, lay, ks, vs, src, dst, is_in)
+            return len(src)
+
+        assert sw.swap_out_seqs([5, 2]) == oracle_swap(ob, ocpu, [5, 2], False) == 21
+        bm.allocate_blocks_for_seqs(_i32([7], cuda), _i32([16 * 5], cuda))     # takes some freed low ids
+        ob.allocate_blocks_for_seqs([7], [16 * 5])
+        assert sw.swap_in_seqs([2, 5]) == oracle_swap(ocpu, ob, [2, 5], True)
+        torch.cuda.synchronize()
+        assert_state_equal(manager_state(bm), ob.snapshot(), "gpu manager")
+        assert_state_equal(manager_state(sw.cpu_block_manager), ocpu.snapshot(), "cpu manager")
+        assert np.array_equal(bits(sw.k_swap), bits(ks)) and np.array_equal(bits(sw.v_swap), bits(vs))
+        blk = lay.block_elems
+        assert np.array_equal(bits(pool.k_cache).reshape(-1), arena[:32 * blk].view(np.uint16))
+        assert np.array_equal(bits(pool.v_cache).reshape(-1), arena[32 * blk:].view(np.uint16))
+    finally:
+        pool.close()
