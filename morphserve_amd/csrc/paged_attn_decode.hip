@@ -626,14 +626,17 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
                           const int32_t* seq_lens, float scale2, int32_t layer,
                           int32_t blocks_per_split, int32_t max_splits, const void* k_new,
                           const void* v_new, const void* cos_t, const void* sin_t) {
-    const bool mfma = g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
+    // the vector-ALU kernel exists for the power-of-two groups only; every other group
+    // size (up to the 16 columns of a matrix tile) runs on the matrix cores
+    constexpr bool has_valu = G == 1 || G == 2 || G == 4 || G == 8;
+    const bool mfma = !has_valu || g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
     if (mfma) {
         hipLaunchKernelGGL(attn_decode_phase1_mfma<G>, grid, dim3(256), 0, s, (const uint4*)q,
                            (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
                            max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
                            max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
                            (const uint4*)sin_t);
-    } else {
+    } else if constexpr (has_valu) {
         hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
                            (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
                            seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
@@ -699,11 +702,16 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
         break;
             MKV_CASE(1)
             MKV_CASE(2)
+            MKV_CASE(3)
             MKV_CASE(4)
+            MKV_CASE(5)
+            MKV_CASE(6)
+            MKV_CASE(7)
             MKV_CASE(8)
+            MKV_CASE(16)
 #undef MKV_CASE
             default:
-                mkv::set_error("unsupported GQA group size %d (supported: 1, 2, 4, 8)", G);
+                mkv::set_error("unsupported GQA group size %d (supported: 1 to 8 and 16)", G);
                 return MKV_EINVAL;
         }
     }

@@ -45,6 +45,21 @@ def _oracle(case, q, layer):
                              case.seq_lens, case.D ** -0.5, layer)
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(6, 2), (5, 1), (12, 2), (28, 4), (32, 2)])
+@pytest.mark.parametrize("target_wgs", [1, 100000])
+def test_decode_attention_other_group_sizes(cuda, Hq, Hkv, target_wgs):
+    """Groups of 3, 5, 6, 7 and 16 query heads per kv head (matrix-core kernel)."""
+    rng = np.random.default_rng(Hq)
+    lens = [1, 16, 17, 100, 1024, 1300]
+    nblk = sum((x + 15) // 16 for x in lens) + 3
+    case = make_case(Hq, 2, Hq, Hkv, lens, num_blocks=nblk, fill="live")
+    q = rand_f16(rng, len(lens), Hq, 128)
+    assert_attn_close(_attend(case, cuda, q, 1, target_wgs=target_wgs), _oracle(case, q, 1), f"G={Hq // Hkv}")
+    with pytest.raises(_capi.MorphKVError, match="group size"):
+        bad = make_case(1, 1, 9, 1, [16], num_blocks=4, fill="live")
+        _attend(bad, cuda, rand_f16(rng, 1, 9, 128), 0)
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(32, 32), (8, 4), (32, 8), (64, 8)])
 @pytest.mark.parametrize("policy", ["auto", "reference"])
 @pytest.mark.parametrize("variant", [1, 2])
@@ -153,7 +168,7 @@ def test_decode_attention_config2_batch_one_layer(cuda):
     assert_attn_close(got, _oracle(case, q, layer), "config 2 batch")
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(32, 32), (32, 8), (64, 8)])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 32), (32, 8), (64, 8), (28, 4), (6, 2), (32, 2)])
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("target_wgs", [1, 100000])
 def test_fused_append_and_attend(cuda, Hq, Hkv, variant, target_wgs):
