@@ -315,6 +315,32 @@ def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, 
             "host_cpu_count": os.cpu_count()}
 
 
+def cpu_baseline_resize(rng):
+    """The oracle's shrink with migration (plan, NumPy block copies, table rewrite) on a pool
+    scaled down to 1536 blocks of the same 2 MiB geometry, 60 % of the kept blocks live."""
+    from oracle import ref_cpu as R
+    L, HKV, D, B = 32, 8, 128, 16
+    total, new_n = 1536, 640
+    lay = R.plain_layout(total, L, HKV, B, D)
+    arena = np.ones(2 * total * lay.block_elems, dtype=np.float16)        # 3 GiB of host memory
+    bm = R.BlockManagerOracle("GPU", total, 64, 64, B)
+    live = rng.permutation(total)[:int(0.6 * new_n)]
+    for s_ in range(len(live) // 48):
+        bm.block_table[s_, :48] = live[s_ * 48:(s_ + 1) * 48]
+        bm.num_seq_allocated_blocks[s_] = 48
+    live = live[:(len(live) // 48) * 48]
+    bm.is_block_free[live] = False
+    bm.num_free_blocks = total - len(live)
+    t0 = time.perf_counter()
+    src, _ = R.apply_migration(arena, lay, bm, new_n)
+    dt = time.perf_counter() - t0
+    moved = len(src) * 2 * lay.block_elems * 2
+    return {"value": round(2 * moved / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{len(src)} moves of 2 MiB blocks out of a {total}-block pool shrunk to {new_n} "
+                      f"({len(live)} live), {dt * 1e3:.0f} ms, NumPy copies on one core",
+            "host_cpu_count": os.cpu_count()}
+
+
 # ---------------------------------------------------------------------------------
 def bench_resize(args):
     import torch
@@ -374,7 +400,11 @@ def bench_resize(args):
     traffic = 2 * moved_bytes                          # read + write
     achieved = traffic / (mg_ms * 1e-3) / 1e9
     whole = traffic / shrink_s / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline_resize(rng)
     return {
+        **({"cpu_baseline": cpu} if cpu else {}),
         "metric": "pool resize + live-block migration HBM GB/s (read+write), 1 MI355X",
         "value": round(whole, 1), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 0,
         "ms_per_step": round(shrink_s * 1e3, 3), "higher_is_better": True, "scaling": "weak",
