@@ -47,6 +47,7 @@ static constexpr int kKBuf = kKTile * kRowBytes;
 static constexpr int kVBuf = kKTile * kRowBytesV;
 static constexpr float kPNegBig = -1.0e30f;
 static constexpr float kPLog2e = 1.442695040888963f;
+static constexpr float kLazyLog2 = 8.0f;    // growth of a row max (in octaves) that forces a rescale
 
 struct PrefillArgs {
     const __half* q;          // [T, Hq, D]
@@ -286,14 +287,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
             for (int n = 0; n < 4; ++n) mx = max3(max3(mx, st[u][n][0], st[u][n][1]), st[u][n][2], st[u][n][3]);
             mx = max_over_groups(mx);
-            if (__ballot(mx > m_run[u]) != 0) {       // some row's max moved: rescale (wave-uniform branch)
+            // m_run is the exponent's reference point, not necessarily the exact running max:
+            // it is moved (and the accumulators rescaled) only when some row's max has grown
+            // by more than kLazyLog2 octaves, so probabilities stay below 2^kLazyLog2 -- well
+            // inside fp16 -- and the final acc / lsum is the same quotient either way.
+            if (__ballot((mx - m_run[u]) * a.scale2 > kLazyLog2) != 0) {      // wave-uniform branch
                 const float alpha = pf_exp2((m_run[u] - mx) * a.scale2);
                 lsum[u] *= alpha;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
+                m_run[u] = mx;
             }
-            m_run[u] = mx;
-            const float ms = -mx * a.scale2;
+            const float ms = -m_run[u] * a.scale2;
             float p[4][4];
 #pragma unroll
             for (int n = 0; n < 4; ++n)

@@ -88,6 +88,34 @@ def test_prefill_attention_parity(cuda, Hq, Hkv, lens):
     assert_attn_close(o.cpu().numpy(), want, f"prefill Hq={Hq} Hkv={Hkv}")
 
 
+@pytest.mark.parametrize("step_octaves", [0.5, 3.0, 20.0])
+def test_prefill_attention_growing_scores(cuda, step_octaves):
+    """Scores that climb along the key axis: the row max keeps moving, by less than, about, or far
+    more than the distance at which the kernel moves its exponent reference and rescales."""
+    rng = np.random.default_rng(5)
+    Hq, Hkv, n = 4, 2, 700
+    q = np.zeros((n, Hq, 128), np.float32)
+    k = np.zeros((n, Hkv, 128), np.float32)
+    q[:, :, 0] = 1.0
+    q[:, :, 1:] = rng.standard_normal((n, Hq, 127)) * 0.05
+    # q.k / sqrt(D) * log2(e) grows by step_octaves every 64 keys, with noise on top
+    ramp = (np.arange(n) // 64) * step_octaves / (128 ** -0.5 * 1.4426950408889634)
+    k[:, :, 0] = ramp[:, None]
+    k[:, :, 1:] = rng.standard_normal((n, Hkv, 127))
+    q, k = q.astype(np.float16), k.astype(np.float16)
+    v = rand_f16(rng, n, Hkv, 128)
+    lens = [n]
+    want = R.prefill_attention(q, k, v, np.array([0]), np.asarray(lens), 128 ** -0.5, math="np32")
+    model = Cfg(num_layers=1, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128)
+    engine = Cfg(block_size=16, max_blocks_per_seq=64)
+    st = build_infer_state(lens, [0], [], Hkv, 128)
+    o = torch.full((n, Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
+    prefill_attention(torch.from_numpy(q).to(cuda), torch.from_numpy(k).to(cuda),
+                      torch.from_numpy(v).to(cuda), o, model, engine, st)
+    torch.cuda.synchronize()
+    assert_attn_close(o.cpu().numpy(), want, f"prefill with scores growing {step_octaves} octaves per tile")
+
+
 def test_chunked_prefill_over_paged_cache(cuda):
     """Second half of each prompt as a chunk whose first half is already cached."""
     rng = np.random.default_rng(77)
