@@ -65,6 +65,23 @@ def test_host_only_entry_points():
         swiftllm_c.replace_layer_org2quant(0)
 
 
+def test_plain_c_program_links_and_calls_the_library(tmp_path):
+    """morphkv.h is valid C99 and a C program (no Python, no torch) links against the library."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    from morphserve_amd import _capi
+    libdir = os.path.dirname(_capi.LIB_PATH)
+    exe = str(tmp_path / "abi_consumer")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "c", "abi_consumer.c"), "-o", exe, "-L", libdir, "-lmorphkv",
+                    "-Wl,-rpath," + libdir], check=True, capture_output=True, text=True)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    assert "abi_consumer: ok" in res.stdout
+
+
 def test_seq_block_size_matches_oracle():
     from morphserve_amd import select_seq_block_size
     rng = np.random.default_rng(0)
