@@ -616,6 +616,68 @@ __global__ __launch_bounds__(128) void attn_decode_phase2(
     o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(ns > 0 ? acc / l : 0.f);
 }
 
+// Phase 2 for many splits (long contexts at small batch): the serial loop above is one
+// dependent chain of loads per thread.  Here a workgroup of four waves takes one
+// (sequence, q head); splits are consumed 64 at a time: every wave reads the chunk's 64
+// log-sum-exps (one per lane), reduces them to the chunk max and the weights
+// w_s = exp2(lse_s - max) -- the same values in all four waves --, then wave w gathers the
+// partials of splits w, w+4, ... with SIXTEEN independent 8-byte loads per lane in flight
+// (lane l owns dims 2l, 2l+1; out-of-range slots re-read the chunk's last split with weight
+// zero).  The four waves' sums meet in LDS.
+__global__ __launch_bounds__(256) void attn_decode_phase2_wide(
+    const float* __restrict__ mid_o, const float* __restrict__ mid_lse, __half* __restrict__ o,
+    const int32_t* __restrict__ seq_lens, int32_t num_q_heads, int32_t tokens_per_split,
+    int32_t max_splits) {
+    __shared__ float part[4][kD];
+    const int i = blockIdx.y;
+    const int hq = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int len = seq_lens[i];
+    const int ns = min((len + tokens_per_split - 1) / tokens_per_split, max_splits);
+    const int64_t base = ((int64_t)i * num_q_heads + hq) * max_splits;
+    float m = kNegBig, l = 0.f, a0 = 0.f, a1 = 0.f;
+    for (int s0 = 0; s0 < ns; s0 += 64) {
+        const int cnt = min(64, ns - s0);
+        const float lse = lane < cnt ? mid_lse[base + s0 + lane] : kNegBig;
+        float mc = lse;
+#pragma unroll
+        for (int sh = 32; sh >= 1; sh >>= 1) mc = fmaxf(mc, __shfl_xor(mc, sh));
+        const float m_new = fmaxf(m, mc);
+        const float old = fast_exp2(m - m_new);
+        const float wgt = lane < cnt ? fast_exp2(lse - m_new) : 0.f;
+        float wsum = wgt;
+#pragma unroll
+        for (int sh = 32; sh >= 1; sh >>= 1) wsum += __shfl_xor(wsum, sh);
+        l = l * old + wsum;
+        a0 *= old;
+        a1 *= old;
+        m = m_new;
+        float2 v[16];
+        float w[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int j = wave + 4 * e;                                // wave-uniform
+            const int jc = min(j, cnt - 1);
+            w[e] = j < cnt ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wgt), jc)) : 0.f;
+            v[e] = *(const float2*)(mid_o + (base + s0 + jc) * kD + 2 * lane);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            a0 = fmaf(w[e], v[e].x, a0);
+            a1 = fmaf(w[e], v[e].y, a1);
+        }
+    }
+    part[wave][2 * lane] = a0;
+    part[wave][2 * lane + 1] = a1;
+    __syncthreads();
+    if (threadIdx.x < kD) {
+        const int d = threadIdx.x;
+        const float acc = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
+        o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(ns > 0 ? acc / l : 0.f);
+    }
+}
+
 // 0: by group size (matrix cores for G >= 4), 1: vector ALU kernel, 2: matrix-core kernel
 static int g_decode_variant = 0;
 
@@ -684,6 +746,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
                 "tokens_per_split %d must be a positive multiple of block_size %d", tokens_per_split, pool->block_size);
     MKV_REQUIRE(max_splits >= 1, "max_splits must be >= 1");
     MKV_REQUIRE(max_splits == 1 || (mid_o && mid_lse), "scratch buffers are NULL");
+    MKV_REQUIRE(((uintptr_t)mid_o & 15) == 0 && ((uintptr_t)mid_lse & 3) == 0, "mid_o must be 16-byte aligned, mid_lse 4-byte aligned");
     MKV_REQUIRE(n <= 65535 && pool->num_kv_heads <= 65535, "grid dimension limit: n, Hkv <= 65535");
     MKV_REQUIRE(((uintptr_t)q & 15) == 0, "q must be 16-byte aligned");
     const int G = num_q_heads / pool->num_kv_heads;
@@ -718,9 +781,15 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
     MKV_HIP(hipGetLastError());
     if (max_splits > 1) {
         mkv::ProfScope prof(MKV_K_ATTN_PHASE2, s);
-        hipLaunchKernelGGL(mkv::attn_decode_phase2, dim3((unsigned)num_q_heads, (unsigned)n),
-                           dim3(128), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
-                           seq_lens, num_q_heads, tokens_per_split, max_splits);
+        if (max_splits > 8) {       // a long chain of partials per head: the gather-in-parallel merge
+            hipLaunchKernelGGL(mkv::attn_decode_phase2_wide, dim3((unsigned)num_q_heads, (unsigned)n),
+                               dim3(256), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
+                               seq_lens, num_q_heads, tokens_per_split, max_splits);
+        } else {
+            hipLaunchKernelGGL(mkv::attn_decode_phase2, dim3((unsigned)num_q_heads, (unsigned)n),
+                               dim3(128), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
+                               seq_lens, num_q_heads, tokens_per_split, max_splits);
+        }
         MKV_HIP(hipGetLastError());
     }
     return MKV_OK;

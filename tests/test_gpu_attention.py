@@ -60,6 +60,21 @@ def test_decode_attention_other_group_sizes(cuda, Hq, Hkv, target_wgs):
         _attend(bad, cuda, rand_f16(rng, 1, 9, 128), 0)
 
 
+@pytest.mark.parametrize("Hq,Hkv,variant", [(8, 2, 0), (4, 4, 1)])
+def test_decode_attention_many_splits(cuda, Hq, Hkv, variant):
+    """Long contexts cut into 47 and 105 splits (more than one 64-split chunk of the merge
+    kernel), next to sequences that use one or two of the launched splits."""
+    rng = np.random.default_rng(11)
+    for lens in ([9000, 300, 5000, 1], [20000, 16, 129]):
+        tps, splits = PA.choose_split(len(lens), Hkv, max(lens), 16, target_wgs=100000)
+        assert splits > 8 and (max(lens) < 10000 or splits > 64)
+        nblk = sum((x + 15) // 16 for x in lens) + 5
+        case = make_case(len(lens), 2, Hq, Hkv, lens, num_blocks=nblk, fill="live")
+        q = rand_f16(rng, len(lens), Hq, 128)
+        assert_attn_close(_attend(case, cuda, q, 1, target_wgs=100000, variant=variant), _oracle(case, q, 1),
+                          f"{splits} splits")
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(32, 32), (8, 4), (32, 8), (64, 8)])
 @pytest.mark.parametrize("policy", ["auto", "reference"])
 @pytest.mark.parametrize("variant", [1, 2])
