@@ -15,8 +15,9 @@ from ... import _capi
 from ._pool import pool_from_args
 
 # Scratch for the per-split partials, grown on demand and reused across calls
-# (the reference allocates it on every call, paged_attn.py:780-793).
-_scratch: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+# (the reference allocates it on every call, paged_attn.py:780-793).  One buffer per
+# (device, stream): calls on one stream are ordered, calls on different streams may overlap.
+_scratch: Dict[Tuple[int, int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
 
 # "auto": split length chosen here for the MI355X grid; "reference": use the
 # caller's infer_state.seq_block_size as the reference kernels do.
@@ -44,7 +45,7 @@ def choose_split(n: int, num_kv_heads: int, max_len: int, block_size: int,
 
 def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
     need_lse = n * hq * splits
-    key = (device.index or 0, d)
+    key = (device.index or 0, _capi.current_stream(), d)
     cur = _scratch.get(key)
     if cur is None or cur[1].numel() < need_lse:
         grow = max(need_lse, 2 * cur[1].numel() if cur else 0)
