@@ -771,10 +771,17 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
             MKV_CASE(6)
             MKV_CASE(7)
             MKV_CASE(8)
+            MKV_CASE(9)
+            MKV_CASE(10)
+            MKV_CASE(11)
+            MKV_CASE(12)
+            MKV_CASE(13)
+            MKV_CASE(14)
+            MKV_CASE(15)
             MKV_CASE(16)
 #undef MKV_CASE
             default:
-                mkv::set_error("unsupported GQA group size %d (supported: 1 to 8 and 16)", G);
+                mkv::set_error("unsupported GQA group size %d (supported: 1 to 16)", G);
                 return MKV_EINVAL;
         }
     }

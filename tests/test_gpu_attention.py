@@ -45,10 +45,11 @@ def _oracle(case, q, layer):
                              case.seq_lens, case.D ** -0.5, layer)
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(6, 2), (5, 1), (12, 2), (28, 4), (32, 2)])
+@pytest.mark.parametrize("Hq,Hkv", [(6, 2), (5, 1), (12, 2), (28, 4), (32, 2), (9, 1), (20, 2), (11, 1), (24, 2), (13, 1),
+                                    (14, 1), (15, 1)])
 @pytest.mark.parametrize("target_wgs", [1, 100000])
 def test_decode_attention_other_group_sizes(cuda, Hq, Hkv, target_wgs):
-    """Groups of 3, 5, 6, 7 and 16 query heads per kv head (matrix-core kernel)."""
+    """Groups of 3, 5, 6, 7 and 9 to 16 query heads per kv head (matrix-core kernel)."""
     rng = np.random.default_rng(Hq)
     lens = [1, 16, 17, 100, 1024, 1300]
     nblk = sum((x + 15) // 16 for x in lens) + 3
@@ -56,8 +57,8 @@ def test_decode_attention_other_group_sizes(cuda, Hq, Hkv, target_wgs):
     q = rand_f16(rng, len(lens), Hq, 128)
     assert_attn_close(_attend(case, cuda, q, 1, target_wgs=target_wgs), _oracle(case, q, 1), f"G={Hq // Hkv}")
     with pytest.raises(_capi.MorphKVError, match="group size"):
-        bad = make_case(1, 1, 9, 1, [16], num_blocks=4, fill="live")
-        _attend(bad, cuda, rand_f16(rng, 1, 9, 128), 0)
+        bad = make_case(1, 1, 17, 1, [16], num_blocks=4, fill="live")
+        _attend(bad, cuda, rand_f16(rng, 1, 17, 128), 0)
 
 
 @pytest.mark.parametrize("Hq,Hkv,variant", [(8, 2, 0), (4, 4, 1)])
