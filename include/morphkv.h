@@ -99,7 +99,9 @@ int mkv_paged_attn_scratch_bytes(int32_t n, int32_t num_q_heads, int32_t head_di
  * A sequence is cut into splits of tokens_per_split tokens (a multiple of the
  * block size); max_splits >= ceil(max_len / tokens_per_split) sizes the scratch
  * rows.  softmax_scale is 1/sqrt(D); the kernel works in base 2. fp32
- * accumulation throughout. */
+ * accumulation throughout.  Limits (MKV_EINVAL otherwise): head_dim 128,
+ * block_size 16, num_q_heads / num_kv_heads from 1 to 16, q 16-byte aligned,
+ * mid_o 16-byte aligned; mid_o / mid_lse may be NULL when max_splits is 1. */
 int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
                           const int32_t* block_table, int64_t max_blocks_per_seq,
                           const int32_t* seq_ids, const int32_t* seq_lens,
