@@ -143,6 +143,11 @@ int mkv_decode_rope_append_attn(const void* k, const void* v, const void* q,
 int mkv_set_decode_variant(int32_t variant);
 
 /* ---- prefill attention -------------------------------------------------- */
+/* Experiments and tests: pin the prefill kernel's workgroup shape.  0 = by the
+ * longest chunk of the call (eight waves / 256 query rows per workgroup from
+ * 3072 tokens, four waves / 128 rows below), 4 or 8 = always that shape. */
+int mkv_set_prefill_variant(int32_t waves);
+
 /* prefill_attention, MS/worker/kernels/prefill_attn.py:9-139, and the live
  * flash_attn_varlen_func call, MS/worker/layers/transformer_layer.py:154-164:
  * causal attention of each prefill sequence over its own contiguous q, k, v.

@@ -37,10 +37,9 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 static constexpr int kPD = 128;             // head dim
 static constexpr int kKTile = 64;           // keys staged per iteration
 static constexpr int kU = 2;                // 16-row column tiles per wave
-static constexpr int kWaves = 4;            // waves per workgroup
-static constexpr int kThreads = 64 * kWaves;
-static constexpr int kQTile = 16 * kU * kWaves;   // query rows per workgroup
-static constexpr int kFetchSteps = (kKTile * 16) / kThreads;   // 16-byte units per thread per K (or V) tile
+// Waves per workgroup is a kernel parameter: 4 (128 query rows, two workgroups per CU) for short
+// prompts, 8 (256 query rows, one workgroup per CU) for long ones, where a K/V tile staged once
+// serves twice the rows and the next-but-one tile is already on its way in a second register set.
 static constexpr int kRowBytes = 272;       // K tile row stride: 256 data + 16 pad -> conflict-free b128 row reads
 static constexpr int kRowBytesV = 288;      // V tile row stride: rows 8 banks apart -> conflict-free transposing reads
 static constexpr int kKBuf = kKTile * kRowBytes;
@@ -65,7 +64,7 @@ struct PrefillArgs {
     int32_t layer;
     float scale2;                 // softmax scale * log2(e), > 0
     int32_t num_seqs;
-    int32_t num_q_tiles;          // ceil(max_len / kQTile)
+    int32_t num_q_tiles;          // ceil(max_len / query rows per workgroup)
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -86,8 +85,13 @@ __device__ __forceinline__ float max_over_groups(float x) {
     auto b = __builtin_amdgcn_permlane32_swap(yi, yi, false, false);
     return fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
 }
-template <bool PAGED>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
+template <bool PAGED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kQTile = 16 * kU * WAVES;                    // query rows per workgroup
+    constexpr int kFetchSteps = (kKTile * 16) / kThreads;      // 16-byte units per thread per K (or V) tile
+    constexpr int kStepRows = kThreads / 16;                   // tile rows covered by one fetch step
+    constexpr int kSets = WAVES == 8 ? 2 : 1;                  // staging register sets = tiles in flight
     __shared__ __attribute__((aligned(16))) char k_lds[2 * kKBuf];
     __shared__ __attribute__((aligned(16))) char v_lds[2 * kVBuf];
 
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     // probabilities are zero); unmapped table entries read as zeros.
     // Contiguous source: one uniform base per (sequence, kv head) plus a 32-bit byte offset
     // per lane that advances by a constant per tile (the launcher bounds len * Hkv * 256).
-    v4u kreg[kFetchSteps], vreg[kFetchSteps];
+    v4u kreg[kSets][kFetchSteps], vreg[kSets][kFetchSteps];
     const uint32_t row_stride = (uint32_t)Hkv * (kPD * 2);
     const char* k_src = PAGED ? nullptr : (const char*)a.k + (start * Hkv + kvh) * (int64_t)(kPD * 2);
     const char* v_src = PAGED ? nullptr : (const char*)a.v + (start * Hkv + kvh) * (int64_t)(kPD * 2);
@@ -195,26 +199,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (PAGED) tile_ids = bt_row[min((key0 >> 4) + (lane & 3), (kv_len - 1) >> 4)];
     };
     load_tile_ids(0);
-    auto fetch_tile = [&](int key0) {
+    auto fetch_tile = [&](int key0, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
             if (PAGED) {
-                const int blk = min((key0 >> 4) + u, (kv_len - 1) >> 4);
-                const int pos = min(key0 + 16 * u + (tid >> 4), kv_len - 1);
-                const int64_t pid = __builtin_amdgcn_readlane(tile_ids, u);
-                kreg[u] = (v4u){0u, 0u, 0u, 0u};
-                vreg[u] = kreg[u];
+                // a step covers kStepRows keys = kStepRows / 16 blocks; a wave's rows lie in one of them
+                const int blk_in_tile = (kStepRows / 16) * u + ((tid >> 4) >> 4);      // wave-uniform
+                const int blk = min((key0 >> 4) + blk_in_tile, (kv_len - 1) >> 4);
+                const int pos = min(key0 + kStepRows * u + (tid >> 4), kv_len - 1);
+                const int64_t pid = __builtin_amdgcn_readlane(tile_ids, __builtin_amdgcn_readfirstlane(blk_in_tile));
+                kreg[SET][u] = (v4u){0u, 0u, 0u, 0u};
+                vreg[SET][u] = kreg[SET][u];
                 if (pid >= 0 && pid < total_blocks) {
                     BlockAddr ba = block_addr(pool, pid, block_bytes);
                     const int64_t head_off = ((int64_t)a.layer * Hkv + kvh) * (int64_t)(16 * kPD * 2);
                     const uint32_t off = (uint32_t)(pos - (blk << 4)) * (kPD * 2) + (tid & 15) * 16;
-                    kreg[u] = *(const v4u*)(ba.k + head_off + off);
-                    vreg[u] = *(const v4u*)(ba.v + head_off + off);
+                    kreg[SET][u] = *(const v4u*)(ba.k + head_off + off);
+                    vreg[SET][u] = *(const v4u*)(ba.v + head_off + off);
                 }
             } else {
-                const uint32_t off = min(next_off + (uint32_t)u * 16u * row_stride, last_off);
-                kreg[u] = *(const v4u*)(k_src + off);
-                vreg[u] = *(const v4u*)(v_src + off);
+                const uint32_t off = min(next_off + (uint32_t)u * (uint32_t)kStepRows * row_stride, last_off);
+                kreg[SET][u] = *(const v4u*)(k_src + off);
+                vreg[SET][u] = *(const v4u*)(v_src + off);
             }
         }
         next_off += kKTile * row_stride;
@@ -222,13 +229,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
     const int k_wr_off = (tid >> 4) * kRowBytes + (tid & 15) * 16;           // + 16u rows
     const int v_wr_off = (tid >> 4) * kRowBytesV + (tid & 15) * 16;
-    auto stage_tile = [&](int buf) {
+    auto stage_tile = [&](int buf, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
         char* kw = k_lds + buf * kKBuf + k_wr_off;
         char* vw = v_lds + buf * kVBuf + v_wr_off;
 #pragma unroll
         for (int u = 0; u < kFetchSteps; ++u) {
-            *(v4u*)(kw + u * (kThreads / 16) * kRowBytes) = kreg[u];
-            *(v4u*)(vw + u * (kThreads / 16) * kRowBytesV) = vreg[u];
+            *(v4u*)(kw + u * kStepRows * kRowBytes) = kreg[SET][u];
+            *(v4u*)(vw + u * kStepRows * kRowBytesV) = vreg[SET][u];
         }
     };
 
@@ -336,13 +344,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     const int num_tiles = (kv_len + kKTile - 1) / kKTile;
     const bool wave_has_rows = r0w < len;
-    fetch_tile(0);
-    stage_tile(0);
-    __syncthreads();
-    for (int it = 0; it + 1 < num_tiles; ++it) {
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, kSets - 1>;       // the same set when there is only one
+    // tile j travels through register set j % kSets; with two sets tile it+2 is requested while tile
+    // it is consumed and tile it+1, requested one iteration earlier, goes to LDS at the end
+    auto iteration = [&](int it, auto cur_set, auto nxt_set) {
         const int buf = it & 1;
         const int key0 = it * kKTile;
-        fetch_tile(key0 + kKTile);                    // in flight during the math below
+        if (kSets == 1) {
+            fetch_tile(key0 + kKTile, nxt_set);       // in flight during the math below
+        } else if (it + 2 < num_tiles) {
+            fetch_tile(key0 + 2 * kKTile, cur_set);   // cur_set's tile went to LDS one iteration ago
+        }
         if (wave_has_rows && key0 <= wave_max_pos) {  // wave-uniform: some row of this wave sees the tile
             if (key0 + kKTile - 1 <= wave_min_pos) {  // every row sees every key (and all keys < kv_len)
                 tile_body(std::false_type{}, buf, key0);
@@ -350,8 +363,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 tile_body(std::true_type{}, buf, key0);
             }
         }
-        stage_tile(buf ^ 1);                          // the other buffer: last read one iteration ago
+        stage_tile(buf ^ 1, nxt_set);                 // the other buffer: last read one iteration ago
         __syncthreads();
+    };
+    fetch_tile(0, Set0{});
+    if (kSets == 2 && num_tiles > 1) fetch_tile(kKTile, Set1{});
+    stage_tile(0, Set0{});
+    __syncthreads();
+    for (int it = 0; it + 1 < num_tiles; it += 2) {
+        iteration(it, Set0{}, Set1{});
+        if (it + 2 < num_tiles) iteration(it + 1, Set1{}, Set0{});
     }
     {   // the last tile holds the workgroup's diagonal: never fully visible to a wave
         const int it = num_tiles - 1;
@@ -377,20 +398,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }   // part
 }
 
+static constexpr int kLongPrompt = 3072;    // longest chunk from which the eight-wave kernel is used
+static int g_prefill_waves = 0;             // 0: by length; 4 or 8: forced (experiments and tests)
+
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
                           int max_len, hipStream_t s) {
     PrefillArgs args = a;
     args.num_seqs = num_seqs;
-    args.num_q_tiles = cdiv(max_len, kQTile);
+    const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (max_len >= kLongPrompt ? 8 : 4);
+    const int q_tile = 16 * kU * waves;
+    args.num_q_tiles = cdiv(max_len, q_tile);
     const int64_t pairs8 = ((int64_t)a.num_q_heads * num_seqs + 7) / 8 * 8;     // pairs padded to the XCD count
     dim3 grid((unsigned)(pairs8 * ((args.num_q_tiles + 1) / 2)));
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
-        if (paged) {
-            hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, dim3(kThreads), 0, s, args, *pool);
+        if (paged && waves == 8) {
+            hipLaunchKernelGGL((prefill_attn_kernel<true, 8>), grid, dim3(512), 0, s, args, *pool);
+        } else if (paged) {
+            hipLaunchKernelGGL((prefill_attn_kernel<true, 4>), grid, dim3(256), 0, s, args, *pool);
+        } else if (waves == 8) {
+            hipLaunchKernelGGL((prefill_attn_kernel<false, 8>), grid, dim3(512), 0, s, args, empty);
         } else {
-            hipLaunchKernelGGL(prefill_attn_kernel<false>, grid, dim3(kThreads), 0, s, args, empty);
+            hipLaunchKernelGGL((prefill_attn_kernel<false, 4>), grid, dim3(256), 0, s, args, empty);
         }
     }
     MKV_HIP(hipGetLastError());
@@ -400,6 +430,12 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
 }  // namespace mkv
 
 extern "C" {
+
+int mkv_set_prefill_variant(int32_t waves) {
+    MKV_REQUIRE(waves == 0 || waves == 4 || waves == 8, "waves must be 0 (by length), 4 or 8");
+    mkv::g_prefill_waves = waves;
+    return MKV_OK;
+}
 
 int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
                      const int32_t* start_locs, const int32_t* seq_lens, int32_t num_seqs,

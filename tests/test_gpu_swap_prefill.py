@@ -6,7 +6,7 @@ import torch
 from oracle import ref_cpu as R
 from helpers import Cfg, assert_attn_close, make_case, rand_f16
 from gpu_helpers import bits, configs, to_gpu
-from morphserve_amd import (build_infer_state, chunked_prefill_attention, prefill_attention,
+from morphserve_amd import (_capi, build_infer_state, chunked_prefill_attention, prefill_attention,
                             store_kvcache, swiftllm_c)
 from test_gpu_append import _segment_setup
 
@@ -114,6 +114,46 @@ def test_prefill_attention_growing_scores(cuda, step_octaves):
                       torch.from_numpy(v).to(cuda), o, model, engine, st)
     torch.cuda.synchronize()
     assert_attn_close(o.cpu().numpy(), want, f"prefill with scores growing {step_octaves} octaves per tile")
+
+
+@pytest.mark.parametrize("waves", [4, 8])
+def test_prefill_attention_both_workgroup_shapes(cuda, waves):
+    """The 128-row and the 256-row workgroup shapes (the second is picked for long prompts) on ragged
+    lengths around their tile edges, contiguous and paged-with-prefix sources."""
+    rng = np.random.default_rng(21)
+    Hq, Hkv = 4, 2
+    lens = np.array([1, 127, 128, 129, 255, 256, 257, 300, 513, 700])
+    T = int(lens.sum())
+    q = rand_f16(rng, T, Hq, 128)
+    k = rand_f16(rng, T, Hkv, 128)
+    v = rand_f16(rng, T, Hkv, 128)
+    starts = np.cumsum(lens) - lens
+    want = R.prefill_attention(q, k, v, starts, lens, 128 ** -0.5, math="np32")
+    case = make_case(21, 2, Hq, Hkv, lens, num_blocks=int(((lens + 15) // 16).sum()) + 2, fill="all")
+    kc, vc, bt = to_gpu(case, cuda)
+    model, engine = configs(case)
+    st = build_infer_state(lens.tolist(), case.seq_ids.tolist(), [], Hkv, 128)
+    _capi.check(_capi.lib().mkv_set_prefill_variant(waves))
+    try:
+        o = torch.full((T, Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
+        prefill_attention(torch.from_numpy(q).to(cuda), torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda),
+                          o, model, engine, st)
+        torch.cuda.synchronize()
+        assert_attn_close(o.cpu().numpy(), want, f"prefill, {waves} waves")
+        store_kvcache(torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda), kc, vc, [], [], bt, model, engine,
+                      st, 0)
+        prefix = lens // 3
+        l2 = lens - prefix
+        q2 = np.concatenate([q[starts[b] + prefix[b]:starts[b] + lens[b]] for b in range(len(lens))])
+        st2 = build_infer_state(l2.tolist(), case.seq_ids.tolist(), [], Hkv, 128)
+        o2 = torch.full((int(l2.sum()), Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
+        chunked_prefill_attention(torch.from_numpy(q2).to(cuda), kc, vc, [], [], bt, model, engine, st2, 0, o2,
+                                  prefix_lens=torch.from_numpy(prefix.astype(np.int32)).to(cuda))
+        torch.cuda.synchronize()
+    finally:
+        _capi.check(_capi.lib().mkv_set_prefill_variant(0))
+    want2 = np.concatenate([want[starts[b] + prefix[b]:starts[b] + lens[b]] for b in range(len(lens))])
+    assert_attn_close(o2.cpu().numpy(), want2, f"chunk over prefix, {waves} waves")
 
 
 def test_chunked_prefill_over_paged_cache(cuda):
