@@ -34,6 +34,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # (profiles/attn_decode_phase1_mfma_cfg2_pmc_traffic.md); counters cannot be
 # collected from inside this process.
 DECODE_TRAFFIC_BYTES_PER_LAUNCH = 343_622_787
+# the same for the migration kernel of cfg3_resize (14 268 moves) and the prefill attention kernel of
+# cfg4_mixed (profiles/pool_migrate_cfg3_and_cfg4_kernels_pmc_traffic.md)
+MIGRATE_CFG3_TRAFFIC_BYTES_PER_LAUNCH = 59_851_535_225
+PREFILL_CFG4_TRAFFIC_BYTES_PER_LAUNCH = 176_927_463
 
 
 class Cfg:
@@ -258,7 +262,8 @@ def bench_decode(args):
         "roofline": {"bound": "hbm", "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH
-                     if (args.workload, num_blocks) == ("cfg2_llama3_8b_decode", 65536) else None,
+                     if (args.workload, num_blocks, args.batch, list(args.ctx), args.tables) ==
+                        ("cfg2_llama3_8b_decode", 65536, 0, [1024, 1536], "permuted") else None,
                      "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
                      "timing": timing, "avg_launch_ms_bracketed": round(bracketed_ms, 5),
                      "algorithmic_bytes_per_launch": attn_bytes,
@@ -420,7 +425,8 @@ def bench_resize(args):
         "pct_of_hbm_peak": round(100 * whole / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_launch_ms": round(mg_ms / max(mg_launches, 1), 4),
+                     "traffic": MIGRATE_CFG3_TRAFFIC_BYTES_PER_LAUNCH if moves == 14268 else None,
+                     "avg_launch_ms": round(mg_ms / max(mg_launches, 1), 4),
                      "algorithmic_bytes_per_launch": traffic},
     }
 
@@ -696,7 +702,8 @@ def bench_mixed(args):
         "rotary_then_store_ms": round(rope_two_ms, 5), "rotary_store_fused_ms": round(rope_fused_ms, 5),
         "rotary_store_fused_GBs": round(rope_bytes / (rope_fused_ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false, 4>", "achieved": round(tflops, 1),
-                     "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4), "traffic": None},
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4),
+                     "traffic": PREFILL_CFG4_TRAFFIC_BYTES_PER_LAUNCH},
     }
 
 
