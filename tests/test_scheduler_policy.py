@@ -187,3 +187,57 @@ def test_give_back_runs_only_in_calls_without_growth_or_swap_in():
     assert len(sin) == 1 and e.give_backs == 0              # a swap-in suppresses the give-back
     batch, sin, sout = s.get_next_batch(e)
     assert not sin and e.give_backs == 2 and s.num_gpu_blocks == 16
+
+
+@pytest.mark.parametrize("seed,quant_serve", [(0, True), (1, True), (2, False), (3, True), (4, False), (5, True)])
+def test_random_serving_run_keeps_the_books(seed, quant_serve):
+    """Random arrivals through the whole policy: every step the queues are disjoint, the running
+    set fits the budget, ids are unique, segments grown and given back balance, arrival order is
+    kept by admission, and every request finishes."""
+    import random
+    rnd = random.Random(seed)
+    seg, layers = 6, 6
+    e = FakeEngine(24, seg, layers=layers, quant_serve=quant_serve, per_step=2)
+    s = e.scheduler
+    all_reqs, admitted_order, pending = [], [], []
+    for _ in range(60):
+        pending.append(Request(prompt_len=rnd.choice([5, 16, 17, 40, 64, 100]), max_output_len=rnd.randint(1, 40)))
+    steps = 0
+    while (pending or s.waiting_q or s.running_q or s.swapped_q) and steps < 5000:
+        steps += 1
+        if pending and rnd.random() < 0.5:
+            burst = [pending.pop() for _ in range(min(len(pending), rnd.randint(1, 4)))]
+            all_reqs.extend(burst)
+            s.on_requests_arrival(burst)
+        # the block manager's free count as the engine would have left it: everything the
+        # running sequences have stored so far is allocated (evicted ones sit in host memory)
+        e.model.gpu_block_manager.num_free_blocks = s.num_gpu_blocks - sum(
+            -(-(r.prompt_len + max(r.output_len - 1, 0)) // 16) for r in s.running_q)
+        given_back_before = e.give_backs
+        batch, sin, sout = s.get_next_batch(e)
+        is_prefill = batch is not s.running_q
+        if is_prefill:
+            assert not sin and not sout
+            admitted_order.extend(batch)
+        for r in batch:                                   # one token per scheduled sequence
+            r.output_len += 1
+        # -- the books ------------------------------------------------------------------
+        running, waiting, swapped = set(map(id, s.running_q)), set(map(id, s.waiting_q)), set(map(id, s.swapped_q))
+        assert not (running & waiting) and not (running & swapped) and not (waiting & swapped)
+        assert len(s.running_q) <= e.engine_config.max_batch_size
+        ids = [r.request_id for r in s.running_q] + [r.request_id for r in s.swapped_q]
+        assert len(ids) == len(set(ids)) and all(0 <= i < e.engine_config.max_seqs_in_block_table for i in ids)
+        if not is_prefill:
+            need = sum(-(-(r.prompt_len + r.output_len - 1) // 16) for r in s.running_q)    # before this step's token
+            # the fit is checked before the give-backs of the same call, which look at the block
+            # manager's free count from before this step's allocations (scheduler.py:75-89, :232-233):
+            # the budget the running set was fitted to is the one before those give-backs
+            assert need <= s.num_gpu_blocks + seg * (e.give_backs - given_back_before)
+        assert s.num_gpu_blocks == 24 + seg * len(e.model.layer_quant_list)
+        assert e.grows - e.give_backs == len(e.model.layer_quant_list) <= layers
+        assert quant_serve or e.grows == 0
+        s.on_batch_finish(batch)
+    assert steps < 5000, "the run did not drain"
+    assert all(r.is_finished() for r in all_reqs) and len(all_reqs) == 60
+    assert [id(r) for r in admitted_order] == [id(r) for r in all_reqs]      # head-of-line order of arrival
+    assert len(s.request_id_manager.available_ids) == e.engine_config.max_seqs_in_block_table
