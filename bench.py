@@ -65,6 +65,8 @@ def parse_args():
     ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
                     help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
                          "benchmark's definition) or in id order (diagnostic only)")
+    ap.add_argument("--vmm-chunk-blocks", type=int, default=64,
+                    help="with --pool-backing vmm: blocks per physical allocation (must divide the pool size)")
     ap.add_argument("--pool-backing", choices=["torch", "vmm"], default="torch",
                     help="decode workloads: the pool is a torch allocation (default) or one tensor over HIP "
                          "virtual memory (VmmKVPool)")
@@ -117,9 +119,10 @@ def bench_decode(args):
     live = perm[:pos].copy()
 
     shape = (num_blocks, L, HKV, B, D)
-    if args.pool_backing == "vmm":                # one tensor over HIP virtual memory, 64-block chunks
+    if args.pool_backing == "vmm":                # one tensor over HIP virtual memory
         from morphserve_amd import VmmKVPool
-        vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, chunk_blocks=64)
+        vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq,
+                             chunk_blocks=args.vmm_chunk_blocks)
         k_cache, v_cache = vmm_pool.k_cache, vmm_pool.v_cache
     else:
         k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
