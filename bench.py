@@ -52,7 +52,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "eviction"])
+                             "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
+                             "eviction"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -848,6 +849,43 @@ def bench_serving(args):
     }
 
 
+def bench_mfma_calibration(args):
+    """What the matrix pipe sustains with nothing else in the way: the prefill kernel's 64 matrix
+    instructions per wave and round, (0) on constant register operands, (1) on N(0,1) register
+    operands, (2) on N(0,1) operands read from LDS in the prefill kernel's fragment pattern."""
+    import ctypes as C
+    import torch
+    from morphserve_amd import _capi
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    data = torch.randn(64 * 1024, dtype=torch.float16, device=dev, generator=g)
+    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    lib = _capi.lib()
+    iters = 2000
+    out = {}
+    for mode, name in ((0, "registers_constant_operands"), (1, "registers_normal_operands"), (2, "lds_normal_operands")):
+        flops = C.c_double(0.0)
+        _capi.check(lib.mkv_diag_mfma_loop(mode, 10, data.data_ptr(), sink.data_ptr(), None, _capi.current_stream()))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(max(args.steps, 1)):
+            _capi.check(lib.mkv_diag_mfma_loop(mode, iters, data.data_ptr(), sink.data_ptr(), C.byref(flops),
+                                               _capi.current_stream()))
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / max(args.steps, 1)
+        out[name] = round(flops.value / (ms * 1e-3) / 1e12, 1)
+    best = out["registers_normal_operands"]
+    return {"metric": "matrix-pipe calibration, v_mfma_f32_16x16x32_f16, TFLOP/s", "value": best, "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": 0, "ms_per_step": None, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+            "config": {"workload": "mfma_calibration: 512 workgroups x 4 waves x 2000 rounds x 64 matrix instructions"},
+            "tflops": out, "published_peak_tflops": 2500.0}
+
+
 def bench_copy_calibration(args):
     """A plain device copy of known size (the migration kernel moving 512 blocks of
     2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
@@ -971,7 +1009,8 @@ def main():
     _capi.lib()
     out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
            "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
-           "copy_calibration": bench_copy_calibration, "eviction": bench_eviction,
+           "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
+           "eviction": bench_eviction,
            "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}[args.workload](args)
     print(json.dumps(out))
 

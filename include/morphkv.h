@@ -335,6 +335,15 @@ int mkv_swap_blocks_device_ids(const int64_t* src_ids, const int64_t* dst_ids, i
 #define MKV_K_SWAP            7
 #define MKV_K_ROPE_STORE      8
 #define MKV_K_COUNT           9
+/* Calibration of the matrix pipe (no counterpart in the reference): `iters` rounds of the prefill
+ * kernel's 64 matrix instructions per wave (v_mfma_f32_16x16x32_f16) on 512 workgroups of four
+ * waves, with nothing else in the loop.  mode 0: operands in registers, constant within an operand; 1: operands in
+ * registers taken from data; 2: operands read from LDS in the prefill kernel's fragment pattern.
+ * data: at least 64 KiB of fp16 values, 16-byte aligned; sink: 512 KiB scratch.  *flops (host,
+ * may be NULL) receives the floating-point operations of the launch. */
+int mkv_diag_mfma_loop(int32_t mode, int32_t iters, const void* data, void* sink, double* flops,
+                       void* stream);
+
 /* When enabled, every launch of the kernels above is bracketed by a
  * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
  * returns the launch count and summed duration since the last reset. */

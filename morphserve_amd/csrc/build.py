@@ -26,6 +26,7 @@ SOURCES = [
     "block_pool.hip",
     "migrate.hip",
     "vmm_arena.hip",
+    "diag.hip",
 ]
 
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32.
