@@ -127,3 +127,51 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_bad_arguments_are_refused_before_any_launch():
+    """Every entry point validates its arguments on the host: NULL pointers, unsupported shapes and
+    out-of-range switches come back as a negative status with a message, without a GPU."""
+    from morphserve_amd import _capi
+    lib = _capi.lib()
+    pool = _capi.MkvPool()                    # all zero: no base pointers, no geometry
+    good = _capi.MkvPool()
+    good.k_base, good.v_base = 1 << 20, 1 << 21
+    good.num_blocks_org, good.num_layers, good.num_kv_heads, good.block_size, good.head_dim = 8, 1, 2, 16, 64
+    P, G = ctypes.byref(pool), ctypes.byref(good)
+    A = 1 << 20                               # an aligned non-NULL address that is never dereferenced
+    calls = {
+        "mkv_append_prefill": (None, None, P, None, 0, None, None, None, 1, 16, 0, None),
+        "mkv_paged_attn_decode": (A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_paged_attn_decode/head_dim": (A, A, G, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_decode_append_attn": (A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_decode_rope_append_attn": (A, A, A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_prefill_attn": (A, A, A, A, A, A, 1, 16, 2, 2, 64, 0.1, None),                  # head_dim 64
+        "mkv_prefill_attn/scale": (A, A, A, A, A, A, 1, 16, 2, 2, 128, 0.0, None),
+        "mkv_prefill_attn_paged": (A, A, P, A, 4, A, A, A, None, 1, 16, 2, 0.1, 0, None),
+        "mkv_pool_migrate": (P, A, A, 1, None),
+        "mkv_fill_zero": (A + 4, 64, None),                                                    # unaligned
+        "mkv_swap_blocks": (None, None, 1, 0, P, None, None, None, None),
+        "mkv_swap_blocks_device_ids": (None, None, 1, 0, P, None, None, 1, None),
+        "mkv_rope_store_kvcache": (None, None, None, None, None, P, None, 4, None, None, None, None, 0, 0, 1, 2, 2,
+                                   128, 0, 1, None),
+        "mkv_bm_allocate": (None, 4, None, 4, None, 8, None, None, 1, 16, None, 0, None, None),
+        "mkv_bm_take_first_free": (None, 8, 1, None, None, None),
+        "mkv_bt_append": (None, 4, None, 4, None, None, None, 0, 1, None),
+        "mkv_bt_release": (None, 4, None, 4, None, 1, None, 8, None, None),
+        "mkv_bt_gather_release": (None, 4, None, 4, None, 1, None, 8, None, 0, None, None),
+        "mkv_bm_count_live": (None, 0, 8, None, None),
+        "mkv_pool_plan_shrink": (None, 8, 4, None, None, 0, None, None, None),
+        "mkv_bt_remap": (None, 4, None, 4, None, 8, None),
+        "mkv_arena_create": (0, 0, None),
+        "mkv_arena_resize": (None, 0),
+        "mkv_set_decode_variant": (99,),
+        "mkv_set_prefill_variant": (5,),
+        "mkv_diag_mfma_loop": (7, 1, None, None, None, None),
+        "mkv_prof_collect": (_capi.K_ROPE_STORE + 1, None, None),
+    }
+    for name, args in calls.items():
+        fn = getattr(lib, name.split("/")[0])
+        rc = fn(*args)
+        assert rc < 0, f"{name} accepted bad arguments (returned {rc})"
+        assert lib.mkv_last_error(), f"{name} failed without a message"
