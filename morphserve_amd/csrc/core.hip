@@ -63,14 +63,14 @@ ProfScope::ProfScope(int id, hipStream_t s) : kernel_id(id), stream(s), rec(null
         delete r;
         return;
     }
-    hipEventRecord(r->start, stream);
+    (void)hipEventRecord(r->start, stream);
     rec = r;
 }
 
 ProfScope::~ProfScope() {
     if (!rec) return;
     ProfRec* r = (ProfRec*)rec;
-    hipEventRecord(r->stop, stream);
+    (void)hipEventRecord(r->stop, stream);
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof[kernel_id].push_back(*r);
     delete r;
@@ -113,8 +113,8 @@ int mkv_prof_reset(void) {
     std::lock_guard<std::mutex> lk(mkv::g_prof_mu);
     for (auto& v : mkv::g_prof) {
         for (auto& r : v) {
-            hipEventDestroy(r.start);
-            hipEventDestroy(r.stop);
+            (void)hipEventDestroy(r.start);
+            (void)hipEventDestroy(r.stop);
         }
         v.clear();
     }
