@@ -109,6 +109,26 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
                           int32_t layer, int32_t tokens_per_split, int32_t max_splits,
                           void* mid_o, void* mid_lse, void* stream);
 
+/* mkv_paged_attn_decode for callers that cannot allocate device memory and have no
+ * workspace to pass: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (which allocates its
+ * partials with torch.empty on every call, MS/worker/kernels/paged_attn.py:780-793).
+ * The split partials (mid_o, mid_lse) live in a 16 MiB array built into the library's
+ * device code, one copy per GPU, held until the process ends; the call performs no
+ * hipMalloc / hipFree and calls no allocating routine.  Same kernels, same results
+ * as mkv_paged_attn_decode.  MKV_EINVAL with a message when
+ * n * num_q_heads * max_splits * (128 + 1) * 4 bytes exceed 16 MiB (max_splits == 1
+ * needs no scratch and always fits).  Every call on a GPU shares that GPU's array:
+ * calls that may overlap on one GPU (different streams, different threads) race;
+ * nothing in it has to start at zero, so nothing is cleared between calls.  The
+ * device current at the call must be the stream's device. */
+int mkv_paged_attn_decode_static(const void* q, void* o, const mkv_pool* pool,
+                                 const int32_t* block_table, int64_t max_blocks_per_seq,
+                                 const int32_t* seq_ids, const int32_t* seq_lens,
+                                 int32_t n, int32_t num_q_heads, float softmax_scale,
+                                 int32_t layer, int32_t tokens_per_split, int32_t max_splits,
+                                 void* stream);
+
 /* store_kvcache (decode rows) + paged_attention of one layer in ONE launch: the
  * call pair of MS/worker/layers/transformer_layer.py:116-126, :181-187 for a
  * decode batch.  k, v : [n, Hkv, D] fp16 is token seq_lens[i]-1 of each

@@ -12,6 +12,8 @@
 #include "common.h"
 #include "rope_math.h"
 
+#include <mutex>
+
 namespace mkv {
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -811,6 +813,53 @@ int mkv_paged_attn_decode(const void* q, void* o, const mkv_pool* pool,
     return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
                        num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
                        mid_lse, nullptr, nullptr, nullptr, nullptr, stream);
+}
+
+// ---- the entry point that allocates nothing ----------------------------------------------
+// Split partials of mkv_paged_attn_decode_static live here instead of in a caller-provided
+// workspace: one array per GPU, held from library load until the process ends.  On the host the
+// array's name is only a handle for hipGetSymbolAddress; kernels receive the device address kept
+// in g_static_scratch[device].
+static constexpr size_t kStaticScratchBytes = 16u << 20;
+static constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::mutex g_static_scratch_mu;
+static void* g_static_scratch[kMaxDevices] = {};
+
+int mkv_paged_attn_decode_static(const void* q, void* o, const mkv_pool* pool,
+                                 const int32_t* block_table, int64_t max_blocks_per_seq,
+                                 const int32_t* seq_ids, const int32_t* seq_lens, int32_t n,
+                                 int32_t num_q_heads, float softmax_scale, int32_t layer,
+                                 int32_t tokens_per_split, int32_t max_splits, void* stream) {
+    MKV_REQUIRE(n >= 0 && num_q_heads > 0 && max_splits >= 1, "bad sizes (n=%d, Hq=%d, max_splits=%d)", n,
+                num_q_heads, max_splits);
+    // mid_o [n, Hq, max_splits, 128] fp32 followed by mid_lse [n, Hq, max_splits] fp32
+    const uint64_t rows = (uint64_t)n * (uint64_t)num_q_heads * (uint64_t)max_splits;
+    const uint64_t mid_o_bytes = rows * mkv::kD * 4;
+    const uint64_t need = max_splits > 1 ? mid_o_bytes + rows * 4 : 0;
+    MKV_REQUIRE(need <= kStaticScratchBytes,
+                "mkv_paged_attn_decode_static: n * num_q_heads * max_splits = %llu rows of split partials need "
+                "%llu bytes, the built-in scratch holds %llu (use mkv_paged_attn_decode with a workspace)",
+                (unsigned long long)rows, (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+    int dev = 0;
+    MKV_HIP(hipGetDevice(&dev));
+    MKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d outside [0, %d)", dev, kMaxDevices);
+    void* base = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_static_scratch_mu);
+        if (g_static_scratch[dev] == nullptr) {       // once per device, with that device current
+            void* p = nullptr;
+            MKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            MKV_REQUIRE(p != nullptr, "hipGetSymbolAddress returned a NULL address for the scratch array");
+            g_static_scratch[dev] = p;
+        }
+        base = g_static_scratch[dev];
+    }
+    void* mid_o = max_splits > 1 ? base : nullptr;
+    void* mid_lse = max_splits > 1 ? (void*)((char*)base + mid_o_bytes) : nullptr;
+    return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n, num_q_heads,
+                       softmax_scale, layer, tokens_per_split, max_splits, mid_o, mid_lse, nullptr, nullptr,
+                       nullptr, nullptr, stream);
 }
 
 int mkv_decode_append_attn(const void* k, const void* v, const void* q, void* o,

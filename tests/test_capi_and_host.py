@@ -144,6 +144,7 @@ def test_bad_arguments_are_refused_before_any_launch():
         "mkv_append_prefill": (None, None, P, None, 0, None, None, None, 1, 16, 0, None),
         "mkv_paged_attn_decode": (A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_paged_attn_decode/head_dim": (A, A, G, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_paged_attn_decode_static/too large": (A, A, G, A, 4, A, A, 64, 64, 0.1, 0, 64, 64, None),
         "mkv_decode_append_attn": (A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_decode_rope_append_attn": (A, A, A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_prefill_attn": (A, A, A, A, A, A, 1, 16, 2, 2, 64, 0.1, None),                  # head_dim 64
