@@ -9,6 +9,7 @@ Drop-in names (reference file each mirrors):
 * ``worker.kernels.block_mgmt.*``                    MorphServe/worker/kernels/block_mgmt.py
 * ``worker.block_manager.BlockManager``              MorphServe/worker/block_manager.py
 * ``worker.infer_state.LlamaInferState``             MorphServe/worker/infer_state.py
+* ``model_config.LlamaModelConfig``                  MorphServe/model_config.py (attention geometry, ``get_kvslot_size``)
 * ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
 * ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
 * ``vmm_pool.VmmKVPool``                             the same pool as ONE tensor over HIP virtual memory
@@ -19,6 +20,7 @@ All compute goes through ``libmorphkv.so`` (hand-written HIP for gfx950) via
 ctypes; nothing here falls back to eager PyTorch.
 """
 from . import _capi  # noqa: F401
+from .model_config import LlamaModelConfig  # noqa: F401
 from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
 from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401

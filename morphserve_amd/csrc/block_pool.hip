@@ -43,19 +43,53 @@ __device__ __forceinline__ int64_t block_excl_scan(int64_t v, int64_t* total, in
     return sm[wave] + inc - v;
 }
 
+// One thread's 16 map bytes starting at b0 (16-byte aligned as an address) as a bit mask: bit k is
+// set when byte b0 + k lies in [lo, hi) and is non-zero (want != 0) or zero (want == 0).  A unit
+// that lies wholly inside the range is one 16-byte load.
+__device__ __forceinline__ uint32_t match_mask16(const uint8_t* map, int64_t b0, int64_t lo, int64_t hi,
+                                                uint8_t want) {
+    if (b0 + kBytesPerThread <= lo || b0 >= hi) return 0u;
+    uint32_t nz = 0u, in = 0xffffu;
+    if (b0 >= lo && b0 + kBytesPerThread <= hi) {
+        const uint4 w = *(const uint4*)(map + b0);
+        const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t t = words[q];
+            t |= t >> 4;
+            t |= t >> 2;
+            t |= t >> 1;
+            t &= 0x01010101u;                                   // one flag per non-zero byte
+            nz |= (((t * 0x01020408u) >> 24) & 0xfu) << (4 * q);
+        }
+    } else {
+        in = 0u;
+#pragma unroll
+        for (int k = 0; k < kBytesPerThread; ++k) {
+            const int64_t b = b0 + k;
+            if (b >= lo && b < hi) {
+                in |= 1u << k;
+                if (map[b] != 0) nz |= 1u << k;
+            }
+        }
+    }
+    return (want != 0 ? nz : ~nz) & in;
+}
+
+// The scans below walk [lo, hi) in tiles of kTileBytes that start at an address multiple of 16, so
+// that every thread's unit can be one aligned 16-byte load whatever lo and the map's own alignment.
+__device__ __forceinline__ int64_t aligned_start(const uint8_t* map, int64_t lo) {
+    return lo - (int64_t)(((uintptr_t)map + (uint64_t)lo) & 15u);
+}
+
 // Counts bytes equal to `want` in map[lo, hi) until at least `limit` are seen
 // (early exit at tile granularity).  All threads must call it.
 __device__ int64_t count_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8_t want,
                                int64_t limit, int64_t* sm) {
     int64_t seen = 0;
-    for (int64_t t0 = lo; t0 < hi && seen < limit; t0 += kTileBytes) {
+    for (int64_t t0 = aligned_start(map, lo); t0 < hi && seen < limit; t0 += kTileBytes) {
         const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
-        int64_t c = 0;
-#pragma unroll
-        for (int k = 0; k < kBytesPerThread; ++k) {
-            const int64_t b = b0 + k;
-            if (b < hi) c += ((map[b] != 0) == (want != 0));
-        }
+        const int64_t c = __popc(match_mask16(map, b0, lo, hi, want));
         int64_t tot;
         block_excl_scan(c, &tot, sm);
         seen += tot;
@@ -69,18 +103,10 @@ __device__ int64_t count_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8
 __device__ void take_bytes(uint8_t* map, int64_t lo, int64_t hi, uint8_t want, uint8_t mark,
                            int64_t n, int64_t* out, int64_t* sm) {
     int64_t base = 0;
-    for (int64_t t0 = lo; t0 < hi && base < n; t0 += kTileBytes) {
+    for (int64_t t0 = aligned_start(map, lo); t0 < hi && base < n; t0 += kTileBytes) {
         const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
-        uint32_t bits = 0;
-        int64_t c = 0;
-#pragma unroll
-        for (int k = 0; k < kBytesPerThread; ++k) {
-            const int64_t b = b0 + k;
-            if (b < hi && ((map[b] != 0) == (want != 0))) {
-                bits |= 1u << k;
-                ++c;
-            }
-        }
+        const uint32_t bits = match_mask16(map, b0, lo, hi, want);
+        const int64_t c = __popc(bits);
         int64_t tot;
         int64_t pos = base + block_excl_scan(c, &tot, sm);
 #pragma unroll
@@ -115,10 +141,10 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
     for (int i = tid; i < batch; i += kScanThreads) {
         const int64_t target = ((int64_t)target_lens[i] + block_size - 1) / block_size;
         const int64_t seq = seq_ids[i];
-        if (seq < 0 || seq >= max_seqs) { s_bad = 2; continue; }
+        if (seq < 0 || seq >= max_seqs) { atomicMax(&s_bad, 2); continue; }
         const int64_t have = n_alloc[seq];
         const int64_t need = target - have;
-        if (target > max_blocks_per_seq) s_bad = 2;       // would not fit the table row
+        if (target > max_blocks_per_seq) atomicMax(&s_bad, 2);   // would not fit the table row
         else if (need < 0) atomicMax(&s_bad, 1);
         my_need += need;
     }
@@ -200,10 +226,11 @@ __global__ __launch_bounds__(kScanThreads) void bt_append_kernel(
         int64_t tot;
         const int64_t start = base + block_excl_scan(need, &tot, sm);
         if (ok && need > 0) {
-            const int64_t fit = min(need, max_blocks_per_seq - have);   // never write past the row
+            // never write past the row, and never count more entries than the row holds
+            const int64_t fit = max((int64_t)0, min(need, max_blocks_per_seq - have));
             int32_t* dst = block_table + seq * max_blocks_per_seq + have;
             for (int64_t x = 0; x < fit; ++x) dst[x] = (int32_t)cand[start + x];
-            n_alloc[seq] = (int32_t)(have + need);
+            n_alloc[seq] = (int32_t)(have + fit);
         }
         base += tot;
     }
@@ -222,7 +249,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_release_kernel(
     for (int i = wave; i < batch; i += kScanWaves) {
         const int64_t seq = seq_ids[i];
         if (seq < 0 || seq >= max_seqs) continue;
-        const int32_t cnt = n_alloc[seq];
+        const int32_t cnt = (int32_t)min((int64_t)n_alloc[seq], max_blocks_per_seq);   // a row holds no more
         const int32_t* row = block_table + seq * max_blocks_per_seq;
         for (int j = lane; j < cnt; j += 64) {
             const int64_t id = row[j];
@@ -249,7 +276,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_gather_release_kernel(
     const int tid = threadIdx.x;
     auto count_of = [&](int i) -> int64_t {
         const int64_t seq = seq_ids[i];
-        return (seq >= 0 && seq < max_seqs) ? (int64_t)n_alloc[seq] : 0;
+        return (seq >= 0 && seq < max_seqs) ? min((int64_t)n_alloc[seq], max_blocks_per_seq) : 0;
     };
     // total first: nothing is modified when it does not fit
     int64_t mine = 0;
@@ -326,7 +353,7 @@ __global__ __launch_bounds__(256) void bt_remap_kernel(int32_t* __restrict__ blo
                                                        const int32_t* __restrict__ remap,
                                                        int64_t num_blocks) {
     for (int64_t row = blockIdx.x; row < max_seqs; row += gridDim.x) {
-        const int32_t cnt = n_alloc[row];
+        const int32_t cnt = (int32_t)min((int64_t)n_alloc[row], max_blocks_per_seq);
         int32_t* r = block_table + row * max_blocks_per_seq;
         for (int j = threadIdx.x; j < cnt; j += blockDim.x) {
             const int32_t id = r[j];

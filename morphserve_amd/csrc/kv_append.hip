@@ -66,6 +66,7 @@ __global__ __launch_bounds__(256) void append_prefill_kernel(
     const int len = seq_lens[b];
     const int t0 = j * pool.block_size;
     if (t0 >= len || h0 >= pool.num_kv_heads) return;
+    if (j >= max_blocks_per_seq) return;                     // beyond the table row: never another sequence's block
     const int nh = min(heads_per_part, pool.num_kv_heads - h0);
     const int ntok = min(pool.block_size, len - t0);
     const int64_t seq = seq_ids[b];
@@ -148,6 +149,9 @@ int mkv_append_prefill(const void* k, const void* v, const mkv_pool* pool,
     MKV_REQUIRE(layer >= 0 && layer < pool->num_layers, "layer %d outside [0, %d)", layer, pool->num_layers);
     MKV_REQUIRE(((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0, "k/v must be 16-byte aligned");
     MKV_REQUIRE(num_seqs <= 65535, "at most 65535 prefill sequences per call");
+    MKV_REQUIRE(mkv::cdiv(max_len, pool->block_size) <= max_blocks_per_seq,
+                "max_len %d needs %d blocks per sequence, a block-table row holds %lld", max_len,
+                mkv::cdiv(max_len, pool->block_size), (long long)max_blocks_per_seq);
     // K and V go to separate workgroups, and the kv heads are cut into parts until the grid
     // has about eight workgroups per compute unit (a part keeps at least one head)
     const int64_t cells = (int64_t)mkv::cdiv(max_len, pool->block_size) * num_seqs * 2;

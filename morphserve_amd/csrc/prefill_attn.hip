@@ -196,7 +196,10 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     // so no fetch ever waits on a table lookup.
     int32_t tile_ids = 0;
     auto load_tile_ids = [&](int key0) {
-        if (PAGED) tile_ids = bt_row[min((key0 >> 4) + (lane & 3), (kv_len - 1) >> 4)];
+        if (PAGED) {      // entries past the table row name no block: they read as zeros, never as a neighbour's row
+            const int idx = min((key0 >> 4) + (lane & 3), (kv_len - 1) >> 4);
+            tile_ids = idx < a.max_blocks_per_seq ? bt_row[idx] : -1;
+        }
     };
     load_tile_ids(0);
     auto fetch_tile = [&](int key0, auto set_tag) {

@@ -18,6 +18,10 @@ from . import _capi
 from .worker.block_manager import BlockManager
 
 
+class PoolTooFullError(RuntimeError):
+    """A shrink was asked for whose live blocks do not fit below the cut; nothing was changed."""
+
+
 class ElasticKVPool:
     """Base pool ``[num_blocks, L, Hkv, B, D]`` (K and V) plus equally sized
     extension segments, with a ``BlockManager`` over the whole id range."""
@@ -118,7 +122,7 @@ class ElasticKVPool:
         """Shrink to ``new_num_blocks`` (base pool plus a whole number of segments),
         first moving every live block with id >= ``new_num_blocks`` into the lowest
         free ids below it and rewriting the block table.  Returns the move lists
-        ``(src, dst)``; raises ``RuntimeError`` (state untouched) when the live
+        ``(src, dst)``; raises ``PoolTooFullError`` (state untouched) when the live
         blocks do not fit."""
         bm = self.block_manager
         s = self.kv_cache_new_block_size
@@ -136,8 +140,8 @@ class ElasticKVPool:
     def _relocate_live_blocks(self, new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
         """Plan (device scan) -> batched block copy -> block-table rewrite, then wait: when
         this returns no live block has an id >= ``new_num_blocks`` and the memory behind
-        those ids is no longer read.  Raises ``RuntimeError`` (state untouched) when the
-        live blocks do not fit below the cut."""
+        those ids is no longer read.  Raises ``PoolTooFullError`` (state untouched) when the
+        live blocks do not fit below the cut; a failing launch raises ``MorphKVError``."""
         bm = self.block_manager
         lib = _capi.lib()
         stream = _capi.current_stream()
@@ -150,7 +154,7 @@ class ElasticKVPool:
                                              remap.data_ptr(), self._result.data_ptr(), stream))
         moves, status, free_below = self._result[:3].tolist()
         if status != 0:
-            raise RuntimeError(f"cannot shrink to {new_num_blocks} blocks: {moves} live blocks to move, "
+            raise PoolTooFullError(f"cannot shrink to {new_num_blocks} blocks: {moves} live blocks to move, "
                                f"{free_below} free below the cut")
         if moves:
             pool = self.descriptor()

@@ -16,7 +16,7 @@ from __future__ import annotations
 
 from typing import Callable, List, Optional
 
-from ..elastic_pool import ElasticKVPool
+from ..elastic_pool import ElasticKVPool, PoolTooFullError
 
 
 class _Model:
@@ -101,7 +101,7 @@ def quant2org_and_update_kvcache(engine: PoolEngine, update_kvcache: bool = True
         else:
             try:
                 src, _ = pool.shrink_to(pool.num_blocks - model.kv_cache_new_block_size)
-            except RuntimeError:
+            except PoolTooFullError:       # does not fit: an ordinary refusal; a failed launch propagates
                 return False
             engine.migrated_blocks += int(src.numel())
         if engine.scheduler is not None:

@@ -99,19 +99,22 @@ class BlockManager:
         batch = seq_ids.shape[0]
         upper = min(int(self.is_block_free.shape[0]), batch * self.block_table.shape[1])
         new_ids = torch.empty(max(upper, 1), dtype=torch.int64, device=dev)
+        # the kernel refuses (and modifies nothing) when the request exceeds this capacity: bounding it by
+        # the host's free counter keeps the device state untouched whenever the call is going to raise
+        cap = min(new_ids.shape[0], int(self.num_free_blocks))
         _capi.check(_capi.lib().mkv_bm_allocate(
             self.num_seq_allocated_blocks.data_ptr(), self.num_seq_allocated_blocks.shape[0],
             self.block_table.data_ptr(), self.block_table.shape[1],
             self.is_block_free.data_ptr(), self.is_block_free.shape[0],
             seq_ids.data_ptr(), target_lens.data_ptr(), batch, self.block_size,
-            new_ids.data_ptr(), new_ids.shape[0], self._result.data_ptr(), _capi.current_stream()))
+            new_ids.data_ptr(), cap, self._result.data_ptr(), _capi.current_stream()))
         total, status, found = self._result[:3].tolist()
         if status == _capi.MKV_EINVAL:
             raise ValueError(f"(On {self.device_name}) a sequence id is outside the block table or a target "
                              f"length needs more than {self.block_table.shape[1]} blocks per sequence")
         assert status != _capi.MKV_ELOGIC, \
             f"(On {self.device_name}) Logic error: Some sequences have more blocks already allocated than needed. seq_ids: {seq_ids}, target_lens: {target_lens}"
-        if status == _capi.MKV_ENOSPC or total > self.num_free_blocks:
+        if status == _capi.MKV_ENOSPC:
             raise RuntimeError(f"No enough free blocks available on {self.device_name} ({self.num_blocks} in total, {self.num_free_blocks} free, {total} requested)")
         if total == 0:
             return torch.empty(0, device=dev, dtype=torch.int64)

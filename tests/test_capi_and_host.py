@@ -142,6 +142,7 @@ def test_bad_arguments_are_refused_before_any_launch():
     A = 1 << 20                               # an aligned non-NULL address that is never dereferenced
     calls = {
         "mkv_append_prefill": (None, None, P, None, 0, None, None, None, 1, 16, 0, None),
+        "mkv_append_prefill/row too short": (A, A, G, A, 4, A, A, A, 1, 16 * 4 + 1, 0, None),
         "mkv_paged_attn_decode": (A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_paged_attn_decode/head_dim": (A, A, G, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_paged_attn_decode_static/too large": (A, A, G, A, 4, A, A, 64, 64, 0.1, 0, 64, 64, None),

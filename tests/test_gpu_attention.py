@@ -1,7 +1,8 @@
 """GPU parity of paged decode attention against the CPU oracle.
 
 Tolerance of the path (fp16 output, fp32 accumulation): every element within
-max-abs 2e-3 or max-rel 1e-2 of the oracle's fp32 torch-CPU result.
+max-abs 2e-3 and, where the oracle's value is at least 0.2 in magnitude, max-rel 1e-2 of the oracle's fp32
+torch-CPU result (``helpers.assert_attn_close``).
 """
 import numpy as np
 import pytest
