@@ -1,0 +1,60 @@
+/*
+ * morphkv_diag -- tuning switches and measurement hooks of libmorphkv.so.
+ *
+ * Nothing here has a counterpart in the reference and nothing here is needed to
+ * use the library: these entries pin a kernel variant for A/B runs and tests,
+ * time individual launches with HIP events, and calibrate the matrix pipe.  The
+ * switches are process-global and not thread-safe; production callers leave
+ * them alone.  The reference-facing boundary is morphkv.h.
+ */
+#ifndef MORPHKV_DIAG_H
+#define MORPHKV_DIAG_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Which phase-1 kernel
+ * mkv_paged_attn_decode launches.  0 = by GQA group size (matrix cores when
+ * Hq/Hkv >= 4, vector ALU otherwise), 1 = vector ALU, 2 = matrix cores. */
+int mkv_set_decode_variant(int32_t variant);
+
+/* Experiments and tests: pin the prefill kernel's workgroup shape.  0 = by the
+ * longest chunk of the call (eight waves / 256 query rows per workgroup from
+ * 3072 tokens, four waves / 128 rows below), 4 or 8 = always that shape. */
+int mkv_set_prefill_variant(int32_t waves);
+
+/* ---- measurement ---------------------------------------------------------- */
+/* Kernel ids for mkv_prof_*. */
+#define MKV_K_APPEND_DECODE   0
+#define MKV_K_APPEND_PREFILL  1
+#define MKV_K_ATTN_PHASE1     2
+#define MKV_K_ATTN_PHASE2     3
+#define MKV_K_MIGRATE         4
+#define MKV_K_PREFILL_ATTN    5
+#define MKV_K_FILL_ZERO       6
+#define MKV_K_SWAP            7
+#define MKV_K_ROPE_STORE      8
+#define MKV_K_COUNT           9
+/* Calibration of the matrix pipe (no counterpart in the reference): `iters` rounds of the prefill
+ * kernel's 64 matrix instructions per wave (v_mfma_f32_16x16x32_f16) on 512 workgroups of four
+ * waves, with nothing else in the loop.  mode 0: operands in registers, constant within an operand; 1: operands in
+ * registers taken from data; 2: operands read from LDS in the prefill kernel's fragment pattern.
+ * data: at least 64 KiB of fp16 values, 16-byte aligned; sink: 512 KiB scratch.  *flops (host,
+ * may be NULL) receives the floating-point operations of the launch. */
+int mkv_diag_mfma_loop(int32_t mode, int32_t iters, const void* data, void* sink, double* flops,
+                       void* stream);
+
+/* When enabled, every launch of the kernels above is bracketed by a
+ * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
+ * returns the launch count and summed duration since the last reset. */
+int mkv_prof_enable(int32_t on);
+int mkv_prof_reset(void);
+int mkv_prof_collect(int32_t kernel_id, int64_t* launches, double* total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MORPHKV_DIAG_H */

@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include "morphkv.h"
+#include "morphkv_diag.h"
 
 namespace mkv {
 

@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include "morphkv.h"
+#include "morphkv_diag.h"
 
 #define CHECK(cond)                                                          \
     do {                                                                     \

@@ -10,13 +10,24 @@ import pytest
 from oracle import ref_cpu as R
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "morphkv.h")
+HEADERS = [os.path.join(ROOT, "include", "morphkv.h"), os.path.join(ROOT, "include", "morphkv_diag.h")]
+DIAG_ONLY = ("mkv_set_decode_variant", "mkv_set_prefill_variant", "mkv_diag_mfma_loop", "mkv_prof_enable",
+             "mkv_prof_reset", "mkv_prof_collect")
 
 
-def _declared():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mkv_[a-z0-9_]+)\s*\(", text)))
+def _declared(headers=HEADERS):
+    names = set()
+    for header in headers:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(mkv_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_the_reference_facing_header_holds_no_tuning_or_measurement_entries():
+    boundary = _declared(HEADERS[:1])
+    for name in DIAG_ONLY:
+        assert name not in boundary and name in _declared(HEADERS[1:])
 
 
 def test_header_declares_the_expected_surface():
