@@ -29,15 +29,21 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
-# HBM bytes per launch of the decode attention kernel on this workload, from the
-# FETCH_SIZE and WRITE_SIZE counters scaled by a device copy of known size
-# (profiles/attn_decode_phase1_mfma_cfg2_pmc_traffic.md); counters cannot be
-# collected from inside this process.
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 343_622_787
-# the same for the migration kernel of cfg3_resize (14 268 moves) and the prefill attention kernel of
-# cfg4_mixed (profiles/pool_migrate_cfg3_and_cfg4_kernels_pmc_traffic.md)
-MIGRATE_CFG3_TRAFFIC_BYTES_PER_LAUNCH = 59_851_535_225
-PREFILL_CFG4_TRAFFIC_BYTES_PER_LAUNCH = 176_927_463
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.md")
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of a workload's dominant kernel, from the committed table of FETCH_SIZE /
+    WRITE_SIZE counter runs (counters cannot be collected from inside this process); None when the
+    table has no row for exactly this workload and arguments."""
+    try:
+        for line in open(TRAFFIC_TABLE):
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) >= 3 and cells[0] == key:
+                return int(cells[2].replace(" ", "").replace(",", ""))
+    except OSError:
+        pass
+    return None
 
 
 class Cfg:
@@ -51,7 +57,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
-                    choices=["cfg2_llama3_8b_decode", "cfg5_codellama34b_decode", "cfg3_resize",
+                    choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
                              "eviction"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
@@ -60,8 +66,11 @@ def parse_args():
                     help="time store_kvcache + paged_attention as two calls per layer (default: the fused "
                          "one-launch-per-layer call)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--ctx", type=int, nargs=2, default=[1024, 1536], metavar=("LO", "HI"),
-                    help="decode workloads: context lengths are uniform in [LO, HI]")
+    ap.add_argument("--ctx", type=int, nargs=2, default=None, metavar=("LO", "HI"),
+                    help="decode workloads: context lengths are uniform in [LO, HI] (default: the workload's, "
+                         "[1024, 1536] or, for cfg1, [64, 512])")
+    ap.add_argument("--no-resize", action="store_true",
+                    help="default workload only: skip the pool-resize measurement that follows the decode one")
     ap.add_argument("--batch", type=int, default=0, help="decode workloads: number of sequences (0 = the workload's)")
     ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
                     help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
@@ -71,8 +80,13 @@ def parse_args():
     ap.add_argument("--pool-backing", choices=["torch", "vmm"], default="torch",
                     help="decode workloads: the pool is a torch allocation (default) or one tensor over HIP "
                          "virtual memory (VmmKVPool)")
+    ap.add_argument("--force-split", type=int, nargs=2, default=None, metavar=("TOKENS", "SPLITS"),
+                    help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
     ap.add_argument("--seed", type=int, default=2)
-    return ap.parse_args()
+    args = ap.parse_args()
+    if args.ctx is None:
+        args.ctx = [64, 512] if args.workload == "cfg1_llama2_7b_layer" else [1024, 1536]
+    return args
 
 
 # ---------------------------------------------------------------------------------
@@ -95,6 +109,10 @@ def bench_decode(args):
         # 48 layers, GQA 64 q / 8 kv heads, batch 128, pool ~200 GB of 3 MiB blocks
         L, HQ, HKV, D, B, N = 48, 64, 8, 128, 16, 128
         default_blocks = 63578
+    elif args.workload == "cfg1_llama2_7b_layer":
+        # one Llama-2-7B-shaped layer: MHA 32 / 32 heads, batch 8, pool of 4096 blocks of 256 KiB (1 GiB)
+        L, HQ, HKV, D, B, N = 1, 32, 32, 128, 16, 8
+        default_blocks = 4096
     else:
         L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
         default_blocks = 65536
@@ -144,6 +162,10 @@ def bench_decode(args):
     model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
     engine = Cfg(block_size=B, max_blocks_per_seq=max_blocks_per_seq)
     st = build_infer_state([], seq_ids.tolist(), lens.tolist(), HKV, D)
+    if args.force_split:
+        from morphserve_amd.worker.kernels import paged_attn as PA
+        PA.SPLIT_POLICY = "reference"
+        st.seq_block_size, st.num_seq_blocks = args.force_split
 
     def step_two_calls():
         for layer in range(L):
@@ -178,14 +200,29 @@ def bench_decode(args):
         torch.cuda.synchronize()
     run = graph.replay if graph is not None else step
 
-    for _ in range(args.warmup):
-        run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def timed_ms(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ms_per_step = timed_ms(run)
+    # the other call shape under the same conditions (a graph of its own), for the record
+    other_graph_ms = None
+    if graph is not None:
+        other()
+        torch.cuda.synchronize()
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2):
+            other()
+        graph2.replay()
+        torch.cuda.synchronize()
+        other_graph_ms = timed_ms(graph2.replay)
+        del graph2
 
     # eager step time too (CPU launch overhead included), and the other call shape, for the record
     reps = max(3, args.steps // 4)
@@ -260,14 +297,24 @@ def bench_decode(args):
                    "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "us_per_step": round(ms_per_step * 1e3, 2),
+        **({"note": "latency-bound: one layer moves a few tens of MB, so a step is a few launch latencies long and "
+                    "the HBM fraction says little; us_per_step is the figure to read"}
+           if args.workload == "cfg1_llama2_7b_layer" else {}),
         "eager_ms_per_step": round(eager_ms, 4),
         ("fused_eager_ms_per_step" if args.unfused else "two_call_eager_ms_per_step"): round(other_ms, 4),
+        ("fused_graph_ms_per_step" if args.unfused else "two_call_graph_ms_per_step"):
+            round(other_graph_ms, 4) if other_graph_ms else None,
+        ("fused_graph_pct_of_hbm_peak" if args.unfused else "two_call_graph_pct_of_hbm_peak"):
+            round(100.0 * step_bytes / (other_graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2) if other_graph_ms else None,
         "step_algorithmic_bytes": step_bytes,
-        "roofline": {"bound": "hbm", "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm",
+                     "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>" if HQ // HKV >= 4 else f"attn_decode_phase1<{HQ // HKV}>",
+                     "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH
-                     if (args.workload, num_blocks, args.batch, list(args.ctx), args.tables) ==
-                        ("cfg2_llama3_8b_decode", 65536, 0, [1024, 1536], "permuted") else None,
+                     "traffic": measured_traffic(
+                         f"{args.workload} pool={num_blocks} batch={N} ctx={args.ctx[0]}-{args.ctx[1]} "
+                         f"tables={args.tables} seed={args.seed}"),
                      "avg_launch_ms": round(phase1_ms, 5), "launches_timed": launches,
                      "timing": timing, "avg_launch_ms_bracketed": round(bracketed_ms, 5),
                      "algorithmic_bytes_per_launch": attn_bytes,
@@ -292,20 +339,28 @@ def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, 
     layer = 0
     threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
-    live_sorted = np.sort(live)
-    renum = {int(b): j for j, b in enumerate(live_sorted)}
-    idx = torch.from_numpy(live_sorted).to(k_cache.device)
-    kl = k_cache[idx, layer].cpu().numpy()          # [nlive, Hkv, B, D]
-    vl = v_cache[idx, layer].cpu().numpy()
-    nlive = len(live_sorted)
-    lay = R.plain_layout(nlive, 1, HKV, B, D)
-    arena = np.concatenate([kl.reshape(-1), vl.reshape(-1)])
-    t2 = table.copy()
-    for s in seq_ids:
-        row = t2[s]
-        for j in range(len(row)):
-            if row[j] >= 0:
-                row[j] = renum[int(row[j])]
+    pool_bytes = 2 * k_cache.numel() * 2
+    full_size = pool_bytes <= (4 << 30)
+    if full_size:
+        # the whole pool on the host, the block table as it is
+        lay = R.plain_layout(k_cache.shape[0], k_cache.shape[1], HKV, B, D)
+        arena = np.concatenate([k_cache.cpu().numpy().reshape(-1), v_cache.cpu().numpy().reshape(-1)])
+        t2 = table.copy()
+    else:
+        live_sorted = np.sort(live)
+        renum = {int(b): j for j, b in enumerate(live_sorted)}
+        idx = torch.from_numpy(live_sorted).to(k_cache.device)
+        kl = k_cache[idx, layer].cpu().numpy()          # [nlive, Hkv, B, D]
+        vl = v_cache[idx, layer].cpu().numpy()
+        nlive = len(live_sorted)
+        lay = R.plain_layout(nlive, 1, HKV, B, D)
+        arena = np.concatenate([kl.reshape(-1), vl.reshape(-1)])
+        t2 = table.copy()
+        for s in seq_ids:
+            row = t2[s]
+            for j in range(len(row)):
+                if row[j] >= 0:
+                    row[j] = renum[int(row[j])]
     qh = q[layer].cpu().numpy()
     kh = k_new[layer].cpu().numpy()
     vh = v_new[layer].cpu().numpy()
@@ -319,8 +374,11 @@ def cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, 
     per_layer = t_total / reps
     return {"value": round(bytes_per_layer / per_layer / 1e9, 3), "unit": "GB/s",
             "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of {L} layers of the same batch ({len(lens)} seqs, ctx {int(min(lens))}-{int(max(lens))}), {reps} repetitions, "
-                      f"{per_layer * 1e3:.1f} ms per layer; x{L} layers = {per_layer * L * 1e3:.0f} ms per step (extrapolated)",
+            "sample": (f"full size: the whole {pool_bytes / 2**30:.1f} GiB pool on the host, all {L} layer(s) of the same batch "
+                       f"({len(lens)} seqs, ctx {int(min(lens))}-{int(max(lens))}), {reps} repetitions, "
+                       f"{per_layer * L * 1e3:.2f} ms per step") if full_size and L == 1 else
+                      (f"1 of {L} layers of the same batch ({len(lens)} seqs, ctx {int(min(lens))}-{int(max(lens))}), {reps} repetitions, "
+                       f"{per_layer * 1e3:.1f} ms per layer; x{L} layers = {per_layer * L * 1e3:.0f} ms per step (extrapolated)"),
             "host_cpu_count": os.cpu_count()}
 
 
@@ -429,7 +487,7 @@ def bench_resize(args):
         "pct_of_hbm_peak": round(100 * whole / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MIGRATE_CFG3_TRAFFIC_BYTES_PER_LAUNCH if moves == 14268 else None,
+                     "traffic": measured_traffic(f"cfg3_resize moves={moves}"),
                      "avg_launch_ms": round(mg_ms / max(mg_launches, 1), 4),
                      "algorithmic_bytes_per_launch": traffic},
     }
@@ -707,7 +765,7 @@ def bench_mixed(args):
         "rotary_store_fused_GBs": round(rope_bytes / (rope_fused_ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false, 4>", "achieved": round(tflops, 1),
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4),
-                     "traffic": PREFILL_CFG4_TRAFFIC_BYTES_PER_LAUNCH},
+                     "traffic": measured_traffic(f"cfg4_mixed prefill=8x512 seed={args.seed}")},
     }
 
 
@@ -1007,11 +1065,25 @@ def main():
         sys.exit(1)
     from morphserve_amd import _capi
     _capi.lib()
-    out = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
-           "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
-           "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
-           "eviction": bench_eviction,
-           "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}[args.workload](args)
+    table = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
+             "cfg1_llama2_7b_layer": bench_decode,
+             "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
+             "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
+             "eviction": bench_eviction,
+             "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}
+    out = table[args.workload](args)
+    if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
+        # the second target of the path in the same process and the same JSON line: the decode pool is gone
+        # (its tensors were locals of bench_decode), the resize workload builds its own
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        r = bench_resize(args)
+        out["resize"] = {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"],
+                         "unit": r["unit"], "ms": r["ms_per_step"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
+                         "moves": r["moves"], "moved_GiB": r["moved_GiB"], "expand_s": r["expand_s"],
+                         "zero_fill_GBs": r["zero_fill_GBs"], "dtype": r["dtype"], "roofline": r["roofline"],
+                         **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})}
     print(json.dumps(out))
 
 
