@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction"])
+                             "eviction", "prefill_shapes"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -82,6 +82,11 @@ def parse_args():
                          "virtual memory (VmmKVPool)")
     ap.add_argument("--force-split", type=int, nargs=2, default=None, metavar=("TOKENS", "SPLITS"),
                     help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
+    ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
+                    help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches")
+    ap.add_argument("--prefill-variants", default="0,4,8",
+                    help="prefill_shapes workload: workgroup shapes to time (0 = the library's own choice by prompt "
+                         "length, 4 = four waves / 128 query rows, 8 = eight waves / 256 query rows)")
     ap.add_argument("--seed", type=int, default=2)
     args = ap.parse_args()
     if args.ctx is None:
@@ -944,6 +949,70 @@ def bench_mfma_calibration(args):
             "tflops": out, "published_peak_tflops": 2500.0}
 
 
+def bench_prefill_shapes(args):
+    """Causal prefill attention over the batch's own contiguous q, k, v (MHA 32 / 32 heads, head_dim 128) for
+    a list of prompt batches and every workgroup shape of the kernel: microseconds per launch and TFLOP/s
+    (causal half, QK^T + PV).  `value` is the library's own choice on the first shape."""
+    import torch
+    from morphserve_amd import _capi
+
+    dev = torch.device("cuda:0")
+    lib = _capi.lib()
+    H, D = 32, 128
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    variants = [int(x) for x in args.prefill_variants.split(",")]
+    rows = {}
+    for shape in args.prefill_shapes.split(","):
+        nseq, ln = (int(x) for x in shape.split("x"))
+        T = nseq * ln
+        q = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+        k = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+        v = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+        starts = torch.arange(nseq, dtype=torch.int32, device=dev) * ln
+        lens = torch.full((nseq,), ln, dtype=torch.int32, device=dev)
+        flops = nseq * H * 4 * D * ln * ln / 2
+        outs, row = {}, {}
+        for var in variants:
+            _capi.check(lib.mkv_set_prefill_variant(var))
+            o = torch.full_like(q, float("nan"))
+
+            def run():
+                _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), starts.data_ptr(),
+                                                 lens.data_ptr(), nseq, ln, H, H, D, D ** -0.5, _capi.current_stream()))
+            for _ in range(max(args.warmup, 1)):
+                run()
+            torch.cuda.synchronize()
+            reps = max(args.steps, 5)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                run()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            outs[var] = o
+            row[f"variant_{var}"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
+                                     "frac_of_2500": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4)}
+        _capi.check(lib.mkv_set_prefill_variant(0))
+        base = outs[variants[0]].float()
+        assert torch.isfinite(base).all()
+        row["max_abs_diff_between_variants"] = max(float((outs[x].float() - base).abs().max()) for x in variants)
+        rows[shape] = row
+    first = rows[args.prefill_shapes.split(",")[0]]
+    best = first[f"variant_{variants[0]}"]
+    return {"metric": "causal prefill attention TFLOP/s (fp16 MFMA, fp32 accumulate), 1 MI355X", "value": best["TFLOPs"],
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": best["us"] / 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
+            "data": "synthetic",
+            "config": {"workload": f"prefill_shapes: MHA 32/32 heads, head_dim 128, prompt batches {args.prefill_shapes}, "
+                                   f"workgroup shapes {args.prefill_variants}"},
+            "shapes": rows,
+            "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel",
+                         "achieved": best["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": round(best["TFLOPs"] / 2500.0, 4), "traffic": None}}
+
+
 def bench_copy_calibration(args):
     """A plain device copy of known size (the migration kernel moving 512 blocks of
     2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
@@ -1069,7 +1138,7 @@ def main():
              "cfg1_llama2_7b_layer": bench_decode,
              "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
-             "eviction": bench_eviction,
+             "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes,
              "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
