@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes"])
+                             "eviction", "prefill_shapes", "placement_probe"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -228,6 +228,23 @@ def bench_decode(args):
         torch.cuda.synchronize()
         other_graph_ms = timed_ms(graph2.replay)
         del graph2
+    # the two-call shape with store_kvcache's decode rows deferred into the paged_attention that follows
+    deferred_graph_ms = None
+    if graph is not None:
+        import morphserve_amd
+        morphserve_amd.enable_deferred_decode_append(True)
+        try:
+            step_two_calls()
+            torch.cuda.synchronize()
+            graph3 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph3):
+                step_two_calls()
+            graph3.replay()
+            torch.cuda.synchronize()
+            deferred_graph_ms = timed_ms(graph3.replay)
+            del graph3
+        finally:
+            morphserve_amd.enable_deferred_decode_append(False)
 
     # eager step time too (CPU launch overhead included), and the other call shape, for the record
     reps = max(3, args.steps // 4)
@@ -312,6 +329,9 @@ def bench_decode(args):
             round(other_graph_ms, 4) if other_graph_ms else None,
         ("fused_graph_pct_of_hbm_peak" if args.unfused else "two_call_graph_pct_of_hbm_peak"):
             round(100.0 * step_bytes / (other_graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2) if other_graph_ms else None,
+        "two_call_deferred_append_graph_ms_per_step": round(deferred_graph_ms, 4) if deferred_graph_ms else None,
+        "two_call_deferred_append_graph_pct_of_hbm_peak":
+            round(100.0 * step_bytes / (deferred_graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2) if deferred_graph_ms else None,
         "step_algorithmic_bytes": step_bytes,
         "roofline": {"bound": "hbm",
                      "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>" if HQ // HKV >= 4 else f"attn_decode_phase1<{HQ // HKV}>",
@@ -1013,6 +1033,108 @@ def bench_prefill_shapes(args):
                          "frac": round(best["TFLOPs"] / 2500.0, 4), "traffic": None}}
 
 
+def bench_placement_probe(args):
+    """Does the rate follow the ALLOCATION?  Four KV pools of 32 GiB in one process, the same config-2 decode
+    batch (same tables, same q / k / v) run on each in turn, twice; then a sequential 1 GiB copy inside each
+    pool (the migration kernel on consecutive block ids: streaming, hardly any address translation).
+    Per pool: microseconds per decode layer and GB/s, copy GB/s.  Under `rocprofv3 --pmc` the decode
+    launches come in groups of 32 * (steps + 1) per (round, pool), in that order."""
+    import ctypes as C
+    import subprocess
+    import torch
+    from morphserve_amd import _capi
+
+    dev = torch.device("cuda:0")
+    L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
+    n_pools, nb = 4, args.pool_blocks or 16384
+    reps = max(args.steps, 1)
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
+    nblk = (lens + B - 1) // B
+    perm = rng.permutation(nb)
+    table = np.full((256, 128), -1, dtype=np.int32)
+    seq_ids = rng.permutation(256)[:N].astype(np.int32)
+    pos = 0
+    for i in range(N):
+        table[seq_ids[i], :nblk[i]] = perm[pos:pos + nblk[i]]
+        pos += nblk[i]
+    bt, ids, ln = (torch.from_numpy(x).to(dev) for x in (table, seq_ids, lens))
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    q = torch.randn((L, N, HQ, D), dtype=torch.float16, device=dev, generator=g)
+    kn = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    vn = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((L, N, HQ, D), dtype=torch.float16, device=dev)
+    lib = _capi.lib()
+    stream = _capi.current_stream()
+    attn_bytes, _ = decode_bytes_per_layer(lens, N, HQ, HKV, D, B)
+    pools = []
+    for _ in range(n_pools):
+        k = torch.zeros((nb, L, HKV, B, D), dtype=torch.float16, device=dev)
+        v = torch.zeros((nb, L, HKV, B, D), dtype=torch.float16, device=dev)
+        pools.append((k, v, _capi.make_pool(k, v)))
+
+    def step(pool):
+        for layer in range(L):
+            _capi.check(lib.mkv_decode_append_attn(
+                kn[layer].data_ptr(), vn[layer].data_ptr(), q[layer].data_ptr(), o[layer].data_ptr(), C.byref(pool),
+                bt.data_ptr(), 128, ids.data_ptr(), ln.data_ptr(), N, HQ, float(D ** -0.5), layer, 1536, 1, None, None,
+                stream))
+
+    def timed(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    out = {"pools": []}
+    decode_us = [[0.0] * n_pools for _ in range(2)]
+    for rnd in range(2):
+        for p, (_, _, pool) in enumerate(pools):
+            decode_us[rnd][p] = timed(lambda: step(pool), reps) / L * 1e3
+    moves = 512
+    src = torch.arange(1024, 1024 + moves, dtype=torch.int64, device=dev)
+    dst = torch.arange(0, moves, dtype=torch.int64, device=dev)
+    moved = moves * 2 * (L * HKV * B * D * 2)
+    for p, (k, v, pool) in enumerate(pools):
+        ms = timed(lambda: _capi.check(lib.mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream)), 5)
+        out["pools"].append({"k_address": hex(k.data_ptr()), "v_address": hex(v.data_ptr()),
+                             "decode_us_per_layer": [round(decode_us[0][p], 2), round(decode_us[1][p], 2)],
+                             "decode_GBs": round(attn_bytes / (decode_us[1][p] * 1e-6) / 1e9, 1),
+                             "sequential_copy_GBs_read_plus_write": round(2 * moved / (ms * 1e-3) / 1e9, 1)})
+    try:          # clocks while the decode kernel runs
+        import threading
+        got = {}
+
+        def ask():
+            r = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=30)
+            card = json.loads(r.stdout)
+            card = card.get("card0", card)
+            got.update({kk: vv for kk, vv in card.items() if "speed" in kk and any(x in kk for x in ("sclk", "mclk", "fclk"))})
+        t = threading.Thread(target=ask)
+        t.start()
+        for _ in range(150):
+            step(pools[0][2])
+        torch.cuda.synchronize()
+        t.join()
+        out["clocks_under_load"] = got
+    except Exception as exc:                                   # the tool is optional
+        out["clocks_under_load"] = {"error": str(exc)[:80]}
+    best = max(x["decode_GBs"] for x in out["pools"])
+    worst = min(x["decode_GBs"] for x in out["pools"])
+    return {"metric": "decode attention GB/s per pool allocation (same batch, one process)", "value": best, "unit": "GB/s",
+            "n_gpus": 1, "steps": reps, "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+            "config": {"workload": f"placement_probe: {n_pools} pools of {nb} blocks ({nb * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB "
+                                   f"each), config-2 decode batch on each, fused launches, eager"},
+            "spread_pct": round(100.0 * (best - worst) / best, 2), **out, "roofline": None}
+
+
 def bench_copy_calibration(args):
     """A plain device copy of known size (the migration kernel moving 512 blocks of
     2 MiB: 1 GiB read, 1 GiB written) -- the yardstick the FETCH_SIZE / WRITE_SIZE
@@ -1138,7 +1260,7 @@ def main():
              "cfg1_llama2_7b_layer": bench_decode,
              "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
-             "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes,
+             "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
              "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:

@@ -24,6 +24,7 @@ from .model_config import LlamaModelConfig  # noqa: F401
 from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
 from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
+from .worker.kernels._deferred import enable_deferred_decode_append, flush as flush_pending_appends  # noqa: F401
 from .worker.kernels.paged_attn import (decode_append_and_attend, decode_rope_append_and_attend,  # noqa: F401
                                         paged_attention)
 from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_attention  # noqa: F401

@@ -16,6 +16,7 @@ import torch
 
 from . import _capi
 from .worker.block_manager import BlockManager
+from .worker.kernels import _deferred
 
 
 class PoolTooFullError(RuntimeError):
@@ -142,6 +143,7 @@ class ElasticKVPool:
         this returns no live block has an id >= ``new_num_blocks`` and the memory behind
         those ids is no longer read.  Raises ``PoolTooFullError`` (state untouched) when the
         live blocks do not fit below the cut; a failing launch raises ``MorphKVError``."""
+        _deferred.flush()
         bm = self.block_manager
         lib = _capi.lib()
         stream = _capi.current_stream()

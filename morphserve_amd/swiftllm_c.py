@@ -17,6 +17,7 @@ from typing import Dict, List, Sequence, Tuple
 import torch
 
 from . import _capi
+from .worker.kernels import _deferred
 from .worker.kernels._pool import pool_strided
 
 _kv_info: Dict[str, int] = {}
@@ -38,6 +39,7 @@ def swap_blocks(source_block_ids: List[int], target_block_ids: List[int], is_swa
     assert len(source_block_ids) == len(target_block_ids)
     pool = _capi.make_pool(k_cache, v_cache)
     n = C.c_int64(0)
+    _deferred.flush()
     _capi.check(_capi.lib().mkv_swap_blocks(
         _ids(source_block_ids), _ids(target_block_ids), len(source_block_ids),
         1 if is_swap_in else 0, C.byref(pool), k_swap.data_ptr(), v_swap.data_ptr(),
@@ -64,6 +66,7 @@ def swap_blocks_new_kv_combined(source_block_ids: List[int], target_block_ids: L
     pool = pool_strided(k_cache, v_cache, k_cache_new, v_cache_new, num_blocks_org,
                         org_layer_param_size, kv_cache_new_block_size, k_cache_element_size, nseg)
     n = C.c_int64(0)
+    _deferred.flush()
     _capi.check(_capi.lib().mkv_swap_blocks(
         _ids(source_block_ids), _ids(target_block_ids), len(source_block_ids),
         1 if is_swap_in else 0, C.byref(pool), k_swap.data_ptr(), v_swap.data_ptr(),

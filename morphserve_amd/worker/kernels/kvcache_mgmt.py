@@ -11,6 +11,7 @@ from typing import List
 import torch
 
 from ... import _capi
+from . import _deferred
 from ._pool import pool_from_args
 
 
@@ -43,6 +44,7 @@ def store_kvcache(
     assert k.dtype == torch.float16 and k_cache.dtype == torch.float16
 
     lib = _capi.lib()
+    _deferred.flush()                   # an append remembered by an earlier call goes out first
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
     stream = _capi.current_stream()
     max_blocks_per_seq = block_table.shape[1]
@@ -58,6 +60,12 @@ def store_kvcache(
     if infer_state.num_decoding_seqs > 0:
         tok_off = infer_state.num_prefill_tokens * row_elems * k.element_size()
         ids_off = infer_state.num_prefill_seqs * infer_state.seq_ids.element_size()
+        if _deferred.ENABLED:           # the paged_attention that follows appends these rows inside its launch
+            _deferred.remember(k, v, k.data_ptr() + tok_off, v.data_ptr() + tok_off, pool,
+                               (k_cache, v_cache, list(k_cache_new), list(v_cache_new)), k_cache, v_cache,
+                               block_table, infer_state, infer_state.seq_ids.data_ptr() + ids_off,
+                               infer_state.num_decoding_seqs, cur_layer)
+            return
         _capi.check(lib.mkv_append_decode(
             k.data_ptr() + tok_off, v.data_ptr() + tok_off, C.byref(pool),
             block_table.data_ptr(), max_blocks_per_seq,

@@ -12,6 +12,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ... import _capi
+from . import _deferred
 from ._pool import pool_from_args
 
 # Scratch for the per-split partials, grown on demand and reused across calls
@@ -93,6 +94,7 @@ def decode_append_and_attend(
     n = infer_state.num_decoding_seqs
     if n == 0:
         return
+    _deferred.flush()
     hq, d = model_config.num_q_heads, model_config.head_dim
     tps, splits = _split_for(infer_state, model_config, engine_config)
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
@@ -136,6 +138,7 @@ def decode_rope_append_and_attend(
     hq, d = model_config.num_q_heads, model_config.head_dim
     assert cos is not None and sin is not None and cos.is_contiguous() and sin.is_contiguous()
     assert cos.dtype == torch.float16 and tuple(cos.shape) == (n, d // 2) == tuple(sin.shape)
+    _deferred.flush()
     tps, splits = _split_for(infer_state, model_config, engine_config)
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
     mid_o, mid_lse = (None, None)
@@ -184,8 +187,18 @@ def paged_attention(
     if splits > 1:
         mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
     ids_off = infer_state.num_prefill_seqs * infer_state.seq_ids.element_size()
+    seq_ids_ptr = infer_state.seq_ids.data_ptr() + ids_off
+    lens_ptr = infer_state.decoding_seq_lens.data_ptr()
+    pending = _deferred.take(k_cache, v_cache, block_table, seq_ids_ptr, lens_ptr, n, cur_layer)
+    if pending is not None:
+        # the decode rows store_kvcache was given for this layer are appended by this launch
+        _capi.check(lib.mkv_decode_append_attn(
+            pending.k_ptr, pending.v_ptr, q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(),
+            block_table.shape[1], seq_ids_ptr, lens_ptr, n, hq, float(infer_state.softmax_scale), cur_layer,
+            tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
+        return
     _capi.check(lib.mkv_paged_attn_decode(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
-        infer_state.seq_ids.data_ptr() + ids_off, infer_state.decoding_seq_lens.data_ptr(),
+        seq_ids_ptr, lens_ptr,
         n, hq, float(infer_state.softmax_scale), cur_layer, tps, splits,
         _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))

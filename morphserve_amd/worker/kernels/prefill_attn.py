@@ -15,6 +15,7 @@ from typing import List, Optional
 import torch
 
 from ... import _capi
+from . import _deferred
 from ._pool import pool_from_args
 
 
@@ -62,6 +63,7 @@ def chunked_prefill_attention(
     if infer_state.num_prefill_seqs == 0:
         return
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
+    _deferred.flush()
     _capi.check(_capi.lib().mkv_prefill_attn_paged(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
         infer_state.seq_ids.data_ptr(), infer_state.prefill_seq_start_locs.data_ptr(),

@@ -16,6 +16,7 @@ from typing import List, Tuple
 import torch
 
 from ... import _capi
+from . import _deferred
 from ._pool import pool_from_args
 
 
@@ -69,6 +70,7 @@ def rotary_embedding_and_store_kvcache(
     assert q.shape[0] == infer_state.num_tokens
     pool = pool_from_args(k_cache, v_cache, k_cache_new, v_cache_new, infer_state)
     st = infer_state
+    _deferred.flush()
     _capi.check(_capi.lib().mkv_rope_store_kvcache(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(), C.byref(pool),
         block_table.data_ptr(), block_table.shape[1], st.seq_ids.data_ptr(),

@@ -20,6 +20,7 @@ import torch
 from .. import _capi, swiftllm_c
 from ..elastic_pool import ElasticKVPool
 from .block_manager import BlockManager
+from .kernels import _deferred
 
 
 class KVSwapper:
@@ -55,6 +56,7 @@ class KVSwapper:
             return 0
         if use_kernel:
             desc = self.pool.descriptor()
+            _deferred.flush()
             _capi.check(_capi.lib().mkv_swap_blocks_device_ids(
                 src_ids.to(torch.int64).data_ptr(), dst_ids.data_ptr(), n, 1 if is_swap_in else 0,
                 C.byref(desc), self.k_swap.data_ptr(), self.v_swap.data_ptr(), self.k_swap.shape[0],
