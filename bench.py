@@ -191,7 +191,8 @@ def bench_decode(args):
     torch.cuda.synchronize()
 
     graph = None
-    if not args.no_graph:
+    # a one-layer step is two or three launches: replaying it as a graph costs more than launching it
+    if not args.no_graph and args.workload != "cfg1_llama2_7b_layer":
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
