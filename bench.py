@@ -1041,7 +1041,6 @@ def bench_placement_probe(args):
     Per pool: microseconds per decode layer and GB/s, copy GB/s.  Under `rocprofv3 --pmc` the decode
     launches come in groups of 32 * (steps + 1) per (round, pool), in that order."""
     import ctypes as C
-    import subprocess
     import torch
     from morphserve_amd import _capi
 
@@ -1108,24 +1107,29 @@ def bench_placement_probe(args):
                              "decode_us_per_layer": [round(decode_us[0][p], 2), round(decode_us[1][p], 2)],
                              "decode_GBs": round(attn_bytes / (decode_us[1][p] * 1e-6) / 1e9, 1),
                              "sequential_copy_GBs_read_plus_write": round(2 * moved / (ms * 1e-3) / 1e9, 1)})
-    try:          # clocks while the decode kernel runs
-        import threading
-        got = {}
+    # clocks while the decode kernel runs, read from sysfs (no child process: a program that has
+    # initialised the GPU must not start another one through fork + exec on some hosts)
+    import glob
+    import threading
+    got = {}
 
-        def ask():
-            r = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=30)
-            card = json.loads(r.stdout)
-            card = card.get("card0", card)
-            got.update({kk: vv for kk, vv in card.items() if "speed" in kk and any(x in kk for x in ("sclk", "mclk", "fclk"))})
-        t = threading.Thread(target=ask)
-        t.start()
-        for _ in range(150):
-            step(pools[0][2])
-        torch.cuda.synchronize()
-        t.join()
-        out["clocks_under_load"] = got
-    except Exception as exc:                                   # the tool is optional
-        out["clocks_under_load"] = {"error": str(exc)[:80]}
+    def ask():
+        for name in ("sclk", "mclk", "fclk"):
+            for path in sorted(glob.glob(f"/sys/class/drm/card*/device/pp_dpm_{name}")):
+                try:
+                    cur = [ln.split(":", 1)[1].strip(" *\n") for ln in open(path) if ln.rstrip().endswith("*")]
+                except OSError:
+                    continue
+                if cur:
+                    got[name] = cur[0]
+                    break
+    t = threading.Thread(target=ask)
+    t.start()
+    for _ in range(150):
+        step(pools[0][2])
+    torch.cuda.synchronize()
+    t.join()
+    out["clocks_under_load"] = got or None
     best = max(x["decode_GBs"] for x in out["pools"])
     worst = min(x["decode_GBs"] for x in out["pools"])
     return {"metric": "decode attention GB/s per pool allocation (same batch, one process)", "value": best, "unit": "GB/s",
