@@ -37,6 +37,7 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 static constexpr int kPD = 128;             // head dim
 static constexpr int kKTile = 64;           // keys staged per iteration
 static constexpr int kU = 2;                // 16-row column tiles per wave
+static constexpr int kVPre = 4;             // V^T fragments requested ahead of the softmax arithmetic
 // Waves per workgroup is a kernel parameter: 4 (128 query rows, two workgroups per CU) for short
 // prompts, 8 (256 query rows, one workgroup per CU) for long ones, where a K/V tile staged once
 // serves twice the rows and the next-but-one tile is already on its way in a second register set.
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int v_rd_off = (4 * c + (m >> 2)) * kRowBytesV + (m & 3) * 8;     // + 16n rows, + 32t bytes
 
     // one 64-key tile against this wave's 32 rows
-    auto tile_body = [&](auto masked_tag, int buf, int key0) {
+    auto tile_body = [&](auto masked_tag, int buf, int key0, const uint4 (&kf_first)[4]) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         const char* k_rd = k_lds + buf * kKBuf + k_rd_off;
         const char* v_rd = v_lds + buf * kVBuf + v_rd_off;
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         v4f st[kU][4];
         uint4 kf[2][4];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) kf[0][x] = ((const uint4*)k_rd)[x];
+        for (int x = 0; x < 4; ++x) kf[0][x] = kf_first[x];
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
             if (n < 3) {
@@ -289,6 +290,18 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
                     }
             }
         }
+        // V^T fragments of the first kVPre products are requested now: their LDS latency passes
+        // under the softmax arithmetic instead of in front of the second matrix phase
+        v8h va_pre[kVPre];
+#pragma unroll
+        for (int t = 0; t < kVPre; ++t) {
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (v4s __attribute__((address_space(3)))*)(v_rd + 32 * t));
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (v4s __attribute__((address_space(3)))*)(v_rd + 16 * kRowBytesV + 32 * t));
+            va_pre[t] = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+        __builtin_amdgcn_sched_barrier(0);
         // ---- online softmax per column tile -----------------------------------------------
         __builtin_amdgcn_s_setprio(0);
         v8h pb[kU][2];                 // P^T as B operand: [pair of sub-tiles] = 8 k-slots
@@ -332,11 +345,16 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
                 lsum[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[u][h], lsum[u], 0, 0, 0);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (v4s __attribute__((address_space(3)))*)(vp + 32 * t));
-                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (v4s __attribute__((address_space(3)))*)(vp + 16 * kRowBytesV + 32 * t));
-                const v8h va = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                v8h va;
+                if (h == 0 && t < kVPre) {
+                    va = va_pre[t];
+                } else {
+                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (v4s __attribute__((address_space(3)))*)(vp + 32 * t));
+                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (v4s __attribute__((address_space(3)))*)(vp + 16 * kRowBytesV + 32 * t));
+                    va = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
 #pragma unroll
                 for (int u = 0; u < kU; ++u)
                     acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][h], acc[u][t], 0, 0, 0);
@@ -351,19 +369,29 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     using Set1 = std::integral_constant<int, kSets - 1>;       // the same set when there is only one
     // tile j travels through register set j % kSets; with two sets tile it+2 is requested while tile
     // it is consumed and tile it+1, requested one iteration earlier, goes to LDS at the end
+    auto first_frags = [&](int buf, uint4 (&out)[4]) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) out[x] = ((const uint4*)(k_lds + buf * kKBuf + k_rd_off))[x];
+    };
     auto iteration = [&](int it, auto cur_set, auto nxt_set) {
         const int buf = it & 1;
         const int key0 = it * kKTile;
+        const bool active = wave_has_rows && key0 <= wave_max_pos;    // wave-uniform: some row of this wave sees the tile
+        // the first K fragments are requested before the address arithmetic of the global fetch,
+        // which then covers their LDS latency
+        uint4 kf_first[4];
+        if (active) first_frags(buf, kf_first);
+        __builtin_amdgcn_sched_barrier(0);
         if (kSets == 1) {
             fetch_tile(key0 + kKTile, nxt_set);       // in flight during the math below
         } else if (it + 2 < num_tiles) {
             fetch_tile(key0 + 2 * kKTile, cur_set);   // cur_set's tile went to LDS one iteration ago
         }
-        if (wave_has_rows && key0 <= wave_max_pos) {  // wave-uniform: some row of this wave sees the tile
+        if (active) {
             if (key0 + kKTile - 1 <= wave_min_pos) {  // every row sees every key (and all keys < kv_len)
-                tile_body(std::false_type{}, buf, key0);
+                tile_body(std::false_type{}, buf, key0, kf_first);
             } else {
-                tile_body(std::true_type{}, buf, key0);
+                tile_body(std::true_type{}, buf, key0, kf_first);
             }
         }
         stage_tile(buf ^ 1, nxt_set);                 // the other buffer: last read one iteration ago
@@ -380,7 +408,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     {   // the last tile holds the workgroup's diagonal: never fully visible to a wave
         const int it = num_tiles - 1;
         const int key0 = it * kKTile;
-        if (wave_has_rows && key0 <= wave_max_pos) tile_body(std::true_type{}, it & 1, key0);
+        if (wave_has_rows && key0 <= wave_max_pos) {
+            uint4 kf_first[4];
+            first_frags(it & 1, kf_first);
+            tile_body(std::true_type{}, it & 1, key0, kf_first);
+        }
         __syncthreads();                              // the next part restages buffer 0
     }
 
