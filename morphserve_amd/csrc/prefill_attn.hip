@@ -433,7 +433,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   }   // part
 }
 
-static constexpr int kLongPrompt = 3072;    // longest chunk from which the eight-wave kernel is used
+static constexpr int kLongPrompt = 2048;    // longest chunk from which the eight-wave kernel is used
 static int g_prefill_waves = 0;             // 0: by length; 4 or 8: forced (experiments and tests)
 
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
