@@ -4,6 +4,8 @@ Every case draws its own shapes: group size, batch, lengths (with the block-boun
 15/16/17 and length 1 mixed in), pool size and permutation, layer, split policy, kernel
 variant.  Attention within max-abs 2e-3 / max-rel 1e-2 of the oracle; appends bit-exact.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -17,6 +19,9 @@ from morphserve_amd.worker.kernels import paged_attn as PA
 
 pytestmark = pytest.mark.gpu
 
+# MORPHKV_RANDOM_CASES_SCALE=k multiplies the number of seeds per test (a one-off soak; the default run keeps 1)
+SCALE = max(1, int(os.environ.get("MORPHKV_RANDOM_CASES_SCALE", "1")))
+
 HEADS = [(1, 1), (4, 4), (4, 2), (8, 2), (6, 2), (8, 1), (16, 2), (5, 1), (7, 1), (16, 1)]
 
 
@@ -28,7 +33,7 @@ def _lens(rng, n, hi):
     return out.astype(np.int64)
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(24 * SCALE))
 def test_random_decode_attention(cuda, seed):
     rng = np.random.default_rng(1000 + seed)
     Hq, Hkv = HEADS[int(rng.integers(len(HEADS)))]
@@ -60,7 +65,7 @@ def test_random_decode_attention(cuda, seed):
                       f"seed {seed}: Hq={Hq} Hkv={Hkv} lens={lens.tolist()} layer={layer}/{L} variant={variant}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(12 * SCALE))
 def test_random_fused_append_and_attend(cuda, seed):
     """One launch appends token len-1 and attends: cache bytes bit-exact, output within tolerance."""
     rng = np.random.default_rng(2000 + seed)
@@ -92,7 +97,7 @@ def test_random_fused_append_and_attend(cuda, seed):
     assert_attn_close(o.cpu().numpy().reshape(n, Hq, 128), want, f"seed {seed}: Hq={Hq} Hkv={Hkv} lens={lens.tolist()}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(12 * SCALE))
 def test_random_prefill_and_chunked_prefill(cuda, seed):
     rng = np.random.default_rng(3000 + seed)
     Hq, Hkv = HEADS[int(rng.integers(len(HEADS)))]
