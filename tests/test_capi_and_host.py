@@ -188,3 +188,31 @@ def test_bad_arguments_are_refused_before_any_launch():
         rc = fn(*args)
         assert rc < 0, f"{name} accepted bad arguments (returned {rc})"
         assert lib.mkv_last_error(), f"{name} failed without a message"
+
+
+def test_model_config_kv_sizes_known_answers(tmp_path):
+    """get_kvslot_size (MorphServe/model_config.py:36-40) on the shapes the benchmarks use: bytes of one
+    token's K and V over all layers, and of one 16-token block."""
+    import json
+
+    import torch
+
+    from morphserve_amd import LlamaModelConfig
+    shapes = {   # name: (config.json fields, kv slot bytes, block bytes)
+        "llama-3-8b": (dict(num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, hidden_size=4096), 131072, 2 << 20),
+        "codellama-34b": (dict(num_hidden_layers=48, num_attention_heads=64, num_key_value_heads=8, hidden_size=8192), 196608, 3 << 20),
+        "llama-2-7b": (dict(num_hidden_layers=32, num_attention_heads=32, hidden_size=4096), 524288, 8 << 20),
+    }
+    for name, (fields, slot, block) in shapes.items():
+        cfg = LlamaModelConfig(dict(fields, model_type="llama"))
+        assert cfg.head_dim == 128, name
+        assert cfg.get_kvslot_size() == slot, name
+        assert cfg.get_kvslot_size(torch.float32) == 2 * slot, name
+        assert cfg.get_block_bytes(16) == block, name
+    d = tmp_path / "m"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(dict(shapes["llama-3-8b"][0], model_type="llama", rope_scaling=None)))
+    cfg = LlamaModelConfig.load_from_model_path(str(d))
+    assert (cfg.num_layers, cfg.num_q_heads, cfg.num_kv_heads, cfg.rope_scaling) == (32, 32, 8, 1.0)
+    with pytest.raises(ValueError):
+        LlamaModelConfig(dict(shapes["llama-2-7b"][0], model_type="gpt2"))
