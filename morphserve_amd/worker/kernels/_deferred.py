@@ -9,7 +9,9 @@ or writes the cache through this package first issues the remembered append as a
 (``flush``), on the stream ``store_kvcache`` was called on.
 
 Off by default: while an append is pending the cache does not hold the new token yet, which a caller
-that inspects the cache tensors directly (not through this package) between the two calls would see.
+that inspects the cache tensors directly (not through this package) between the two calls would see,
+and the decode rows of ``k`` and ``v`` are read when the append is finally issued, so they must not be
+overwritten before the attention call (or ``flush_pending_appends()``).
 ``MORPHKV_DEFER_DECODE_APPEND=1`` or ``enable_deferred_decode_append(True)`` turns it on.
 """
 from __future__ import annotations
