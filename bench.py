@@ -84,6 +84,9 @@ def parse_args():
                     help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches")
+    ap.add_argument("--prefill-data", choices=["randn", "zeros"], default="randn",
+                    help="prefill_shapes workload: N(0,1) inputs (default) or all-zero inputs -- the same instruction "
+                         "stream without switching activity in the matrix pipe, to show what the power limit costs")
     ap.add_argument("--prefill-variants", default="0,4,8",
                     help="prefill_shapes workload: workgroup shapes to time (0 = the library's own choice by prompt "
                          "length, 4 = four waves / 128 query rows, 8 = eight waves / 256 query rows)")
@@ -996,9 +999,12 @@ def bench_prefill_shapes(args):
     for shape in args.prefill_shapes.split(","):
         nseq, ln = (int(x) for x in shape.split("x"))
         T = nseq * ln
-        q = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
-        k = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
-        v = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+        if args.prefill_data == "zeros":
+            q, k, v = (torch.zeros((T, H, D), dtype=torch.float16, device=dev) for _ in range(3))
+        else:
+            q = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+            k = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
+            v = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
         starts = torch.arange(nseq, dtype=torch.int32, device=dev) * ln
         lens = torch.full((nseq,), ln, dtype=torch.int32, device=dev)
         flops = nseq * H * 4 * D * ln * ln / 2
@@ -1046,7 +1052,7 @@ def bench_prefill_shapes(args):
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
             "data": "synthetic",
             "config": {"workload": f"prefill_shapes: MHA 32/32 heads, head_dim 128, prompt batches {args.prefill_shapes}, "
-                                   f"workgroup shapes {args.prefill_variants}"},
+                                   f"workgroup shapes {args.prefill_variants}, inputs {args.prefill_data}"},
             "shapes": rows,
             "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel",
                          "achieved": best["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
