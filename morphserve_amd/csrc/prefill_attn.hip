@@ -310,12 +310,15 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             float mx = m_run[u];
 #pragma unroll
             for (int n = 0; n < 4; ++n) mx = max3(max3(mx, st[u][n][0], st[u][n][1]), st[u][n][2], st[u][n][3]);
-            mx = max_over_groups(mx);
             // m_run is the exponent's reference point, not necessarily the exact running max:
             // it is moved (and the accumulators rescaled) only when some row's max has grown
             // by more than kLazyLog2 octaves, so probabilities stay below 2^kLazyLog2 -- well
             // inside fp16 -- and the final acc / lsum is the same quotient either way.
+            // Some row has outgrown the reference iff some LANE's own scores have, so the test
+            // runs on the lane-local max and the row max is completed across the four lane
+            // groups only when the reference does move.
             if (__ballot((mx - m_run[u]) * a.scale2 > kLazyLog2) != 0) {      // wave-uniform branch
+                mx = max_over_groups(mx);
                 const float alpha = pf_exp2((m_run[u] - mx) * a.scale2);
                 lsum[u] *= alpha;
 #pragma unroll
