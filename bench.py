@@ -451,6 +451,15 @@ def bench_resize(args):
     L, HKV, D, B = 32, 8, 128, 16
     ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1          # 32k -> 96k -> 40k blocks of 2 MiB
     rng = np.random.default_rng(args.seed)
+    # one small resize first: a kernel's first launch in a process loads its code object (a few hundred
+    # microseconds each for the plan, copy and table-rewrite kernels), which is not part of a resize
+    small = ElasticKVPool(64, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=64)
+    small.expand(64)
+    small.block_manager.allocate_blocks_for_seqs(torch.arange(4, dtype=torch.int32, device=dev),
+                                                 torch.full((4,), 24 * B, dtype=torch.int32, device=dev))
+    small.block_manager.free_blocks_for_seqs(torch.arange(3, dtype=torch.int32, device=dev))
+    small.shrink_to(64)
+    del small
     pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256)
     blk_bytes = pool.block_bytes
     _capi.prof_reset()
