@@ -442,6 +442,21 @@ def cpu_baseline_resize(rng):
 
 
 # ---------------------------------------------------------------------------------
+def _warm_resize_kernels(dev, L, HKV, B, D):
+    """One small resize with live blocks above the cut: a kernel's first launch in a process loads its code
+    object (a few hundred microseconds each for the plan, copy and table-rewrite kernels), which is not part of
+    a resize."""
+    import torch
+    from morphserve_amd import ElasticKVPool
+    small = ElasticKVPool(64, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=64)
+    small.expand(64)
+    small.block_manager.allocate_blocks_for_seqs(torch.arange(4, dtype=torch.int32, device=dev),
+                                                 torch.full((4,), 24 * B, dtype=torch.int32, device=dev))
+    small.block_manager.free_blocks_for_seqs(torch.arange(3, dtype=torch.int32, device=dev))
+    src, _ = small.shrink_to(64)
+    assert src.numel() == 24
+
+
 def bench_resize(args):
     import torch
     from morphserve_amd import ElasticKVPool, _capi
@@ -451,15 +466,7 @@ def bench_resize(args):
     L, HKV, D, B = 32, 8, 128, 16
     ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1          # 32k -> 96k -> 40k blocks of 2 MiB
     rng = np.random.default_rng(args.seed)
-    # one small resize first: a kernel's first launch in a process loads its code object (a few hundred
-    # microseconds each for the plan, copy and table-rewrite kernels), which is not part of a resize
-    small = ElasticKVPool(64, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=64)
-    small.expand(64)
-    small.block_manager.allocate_blocks_for_seqs(torch.arange(4, dtype=torch.int32, device=dev),
-                                                 torch.full((4,), 24 * B, dtype=torch.int32, device=dev))
-    small.block_manager.free_blocks_for_seqs(torch.arange(3, dtype=torch.int32, device=dev))
-    small.shrink_to(64)
-    del small
+    _warm_resize_kernels(dev, L, HKV, B, D)
     pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256)
     blk_bytes = pool.block_bytes
     _capi.prof_reset()
@@ -548,6 +555,7 @@ def bench_pressure_shrink(args):
     lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     max_seqs, max_bps = 256, 128
+    _warm_resize_kernels(dev, L, HKV, B, D)
     pool = ElasticKVPool(KEEP, L, HKV, B, D, max_seqs_in_block_table=max_seqs, max_blocks_per_seq=max_bps)
     pool.expand(SEG)
     perm = rng.permutation(total)
