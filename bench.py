@@ -84,6 +84,9 @@ def parse_args():
                     help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches")
+    ap.add_argument("--probe-clock-steps", type=int, default=150,
+                    help="placement_probe workload: decode steps run while the clocks are sampled (0 keeps a counter "
+                         "run down to the per-pool launches)")
     ap.add_argument("--prefill-data", choices=["randn", "zeros"], default="randn",
                     help="prefill_shapes workload: N(0,1) inputs (default) or all-zero inputs -- the same instruction "
                          "stream without switching activity in the matrix pipe, to show what the power limit costs")
@@ -1173,7 +1176,7 @@ def bench_placement_probe(args):
                     break
     t = threading.Thread(target=ask)
     t.start()
-    for _ in range(150):
+    for _ in range(args.probe_clock_steps):
         step(pools[0][2])
     torch.cuda.synchronize()
     t.join()
