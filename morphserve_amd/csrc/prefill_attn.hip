@@ -66,6 +66,7 @@ struct PrefillArgs {
     float scale2;                 // softmax scale * log2(e), > 0
     int32_t num_seqs;
     int32_t num_q_tiles;          // ceil(max_len / query rows per workgroup)
+    int32_t pair_tiles;           // 1: a workgroup takes two query tiles (i-th from the end, i-th from the start); 0: one
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -112,9 +113,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int Hq = a.num_q_heads;
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    const int half_tiles = (a.num_q_tiles + 1) >> 1;
-    const int ti = slot % half_tiles;
-    const int pair = (slot / half_tiles) * 8 + xcd;
+    // (When pairing would leave CUs short of workgroups the launcher turns it off: one tile per
+    // workgroup, the longest tiles at the lowest ids so that they start first.)
+    const int slots_per_pair = a.pair_tiles ? (a.num_q_tiles + 1) >> 1 : a.num_q_tiles;
+    const int ti = slot % slots_per_pair;
+    const int pair = (slot / slots_per_pair) * 8 + xcd;
     if (pair >= Hq * a.num_seqs) return;
     const int hq = pair % Hq;
     const int b = pair / Hq;
@@ -123,13 +126,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 
     const int len = a.seq_lens[b];
     const int n_qt = (len + kQTile - 1) / kQTile;            // query tiles of THIS sequence
-    if (2 * ti >= n_qt) return;
+    if ((a.pair_tiles ? 2 * ti : ti) >= n_qt) return;
     const int64_t start = a.start_locs[b];
     const int prefix = (PAGED && a.prefix_lens) ? a.prefix_lens[b] : 0;
 
   for (int part = 0; part < 2; ++part) {
     const int qt = part == 0 ? n_qt - 1 - ti : ti;
-    if (part == 1 && 2 * ti == n_qt - 1) break;              // odd count: the middle tile was part 0
+    if (part == 1 && (!a.pair_tiles || 2 * ti == n_qt - 1)) break;   // unpaired, or odd count: the middle tile was part 0
     const int q0 = qt * kQTile;
     const int kv_len = prefix + min(len, q0 + kQTile);       // keys this workgroup can see
 
@@ -438,16 +441,25 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 
 static constexpr int kLongPrompt = 2048;    // longest chunk from which the eight-wave kernel is used
 static int g_prefill_waves = 0;             // 0: by length; 4 or 8: forced (experiments and tests)
+static int g_prefill_pairing = 0;           // 0: by grid size; 1: always two tiles per workgroup; 2: never
 
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
                           int max_len, hipStream_t s) {
     PrefillArgs args = a;
     args.num_seqs = num_seqs;
-    const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (max_len >= kLongPrompt ? 8 : 4);
+    const int64_t pairs8 = ((int64_t)a.num_q_heads * num_seqs + 7) / 8 * 8;     // pairs padded to the XCD count
+    // eight waves only where their workgroups (one per CU) still cover the chip
+    const bool long_and_wide = max_len >= kLongPrompt && pairs8 * ((cdiv(max_len, 16 * kU * 8) + 1) / 2) >= 256;
+    const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (long_and_wide ? 8 : 4);
     const int q_tile = 16 * kU * waves;
     args.num_q_tiles = cdiv(max_len, q_tile);
-    const int64_t pairs8 = ((int64_t)a.num_q_heads * num_seqs + 7) / 8 * 8;     // pairs padded to the XCD count
-    dim3 grid((unsigned)(pairs8 * ((args.num_q_tiles + 1) / 2)));
+    // two tiles per workgroup balance the causal triangle; a grid that then has fewer workgroups than the
+    // chip has CUs, or a sequence of at most three tiles (little to balance) on a grid below two per CU,
+    // is better off with one tile per workgroup (8 x 256: 21.0 -> 18.6 us, 1 x 1024: 32.7 -> 27.6 us)
+    const int64_t paired = pairs8 * ((args.num_q_tiles + 1) / 2);
+    const bool unpair = paired < 256 || (args.num_q_tiles <= 3 && paired < 512);
+    args.pair_tiles = (g_prefill_pairing == 1 || (g_prefill_pairing == 0 && !unpair)) ? 1 : 0;
+    dim3 grid((unsigned)(args.pair_tiles ? paired : pairs8 * args.num_q_tiles));
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
@@ -470,8 +482,11 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
 extern "C" {
 
 int mkv_set_prefill_variant(int32_t waves) {
+    const int pairing = (waves >> 8) & 3;       // bits 8-9: 0 tiles paired by grid size, 1 always, 2 never
+    waves &= 0xFF;
     MKV_REQUIRE(waves == 0 || waves == 4 || waves == 8, "waves must be 0 (by length), 4 or 8");
     mkv::g_prefill_waves = waves;
+    mkv::g_prefill_pairing = pairing;
     return MKV_OK;
 }
 

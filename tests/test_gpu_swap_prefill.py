@@ -116,10 +116,11 @@ def test_prefill_attention_growing_scores(cuda, step_octaves):
     assert_attn_close(o.cpu().numpy(), want, f"prefill with scores growing {step_octaves} octaves per tile")
 
 
-@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("waves", [4, 8, 4 | (1 << 8), 4 | (2 << 8), 8 | (1 << 8), 8 | (2 << 8)])
 def test_prefill_attention_both_workgroup_shapes(cuda, waves):
     """The 128-row and the 256-row workgroup shapes (the second is picked for long prompts) on ragged
-    lengths around their tile edges, contiguous and paged-with-prefix sources."""
+    lengths around their tile edges, contiguous and paged-with-prefix sources; bits 8-9 of the switch force two
+    query tiles per workgroup (1) or one (2), which the library otherwise chooses by grid size."""
     rng = np.random.default_rng(21)
     Hq, Hkv = 4, 2
     lens = np.array([1, 127, 128, 129, 255, 256, 257, 300, 513, 700])
