@@ -113,11 +113,23 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int Hq = a.num_q_heads;
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    // (When pairing would leave CUs short of workgroups the launcher turns it off: one tile per
-    // workgroup, the longest tiles at the lowest ids so that they start first.)
-    const int slots_per_pair = a.pair_tiles ? (a.num_q_tiles + 1) >> 1 : a.num_q_tiles;
-    const int ti = slot % slots_per_pair;
-    const int pair = (slot / slots_per_pair) * 8 + xcd;
+    // When pairing would leave CUs short of workgroups the launcher turns it off: one tile per
+    // workgroup.  An XCD hands consecutive workgroups to its 32 CUs in turn, so slots s and s + 32
+    // share a CU: the XCD's (tile rank, pair) jobs, longest tiles first, are dealt to the slots in
+    // snake order (every second run of 32 reversed), which puts a long and a short tile on each CU.
+    int ti, pair;
+    if (a.pair_tiles) {
+        const int half_tiles = (a.num_q_tiles + 1) >> 1;
+        ti = slot % half_tiles;
+        pair = (slot / half_tiles) * 8 + xcd;
+    } else {
+        const int pairs_x = (Hq * a.num_seqs + 7) >> 3;
+        const int run = slot >> 5, c32 = slot & 31;
+        const int job = (run << 5) + ((run & 1) ? 31 - c32 : c32);
+        ti = job / pairs_x;
+        pair = (job - ti * pairs_x) * 8 + xcd;
+        if (ti >= a.num_q_tiles) return;
+    }
     if (pair >= Hq * a.num_seqs) return;
     const int hq = pair % Hq;
     const int b = pair / Hq;
@@ -453,13 +465,15 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
     const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (long_and_wide ? 8 : 4);
     const int q_tile = 16 * kU * waves;
     args.num_q_tiles = cdiv(max_len, q_tile);
-    // two tiles per workgroup balance the causal triangle; a grid that then has fewer workgroups than the
-    // chip has CUs, or a sequence of at most three tiles (little to balance) on a grid below two per CU,
-    // is better off with one tile per workgroup (8 x 256: 21.0 -> 18.6 us, 1 x 1024: 32.7 -> 27.6 us)
+    // two tiles per workgroup balance the causal triangle inside a workgroup; a grid that then has fewer
+    // workgroups than the chip holds at once (two per CU), or sequences of at most three tiles, are better off
+    // with one tile per workgroup and the balance made across the two workgroups of a CU
+    // (4 x 512: 25.7 -> 22.4 us, 3 x 700: 39.0 -> 26.1 us, 1 x 1024: 32.5 -> 27.2 us, 8 x 256: 22.0 -> 18.9 us)
     const int64_t paired = pairs8 * ((args.num_q_tiles + 1) / 2);
-    const bool unpair = paired < 256 || (args.num_q_tiles <= 3 && paired < 512);
+    const bool unpair = paired < 512 || args.num_q_tiles <= 3;
     args.pair_tiles = (g_prefill_pairing == 1 || (g_prefill_pairing == 0 && !unpair)) ? 1 : 0;
-    dim3 grid((unsigned)(args.pair_tiles ? paired : pairs8 * args.num_q_tiles));
+    const int64_t unpaired = ((pairs8 / 8 * args.num_q_tiles + 31) / 32 * 32) * 8;      // whole runs of 32 slots per XCD
+    dim3 grid((unsigned)(args.pair_tiles ? paired : unpaired));
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
