@@ -84,6 +84,9 @@ def parse_args():
                     help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches")
+    ap.add_argument("--seq-order", choices=["drawn", "snake"], default="drawn",
+                    help="decode workloads, diagnostic: keep the drawn order of context lengths, or hand the batch over "
+                         "sorted so that slots 256 / Hkv apart (the two workgroups of a CU) hold a long and a short one")
     ap.add_argument("--probe-clock-steps", type=int, default=150,
                     help="placement_probe workload: decode steps run while the clocks are sampled (0 keeps a counter "
                          "run down to the per-pool launches)")
@@ -109,6 +112,11 @@ def decode_bytes_per_layer(lens, n, hq, hkv, d, b):
     return attn, append
 
 
+def _balanced_order():
+    from morphserve_amd.worker.kernels import paged_attn as PA
+    return bool(PA.BALANCED_ORDER)
+
+
 def bench_decode(args):
     import torch
     from morphserve_amd import (_capi, build_infer_state, decode_append_and_attend, paged_attention,
@@ -131,6 +139,14 @@ def bench_decode(args):
     if args.batch:
         N = args.batch
     lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
+    if args.seq_order == "snake":                 # diagnostic: the batch arrives with long and short sequences alternating
+        run = max(1, 256 // HKV)                  # in runs of 256 / Hkv slots, the order that puts one of each on a CU
+        srt = np.sort(lens)[::-1]
+        out = srt.copy()
+        for r in range(len(srt) // run):
+            if r & 1:
+                out[r * run:(r + 1) * run] = srt[r * run:(r + 1) * run][::-1]
+        lens = out.astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     num_blocks = args.pool_blocks or default_blocks
     max_blocks_per_seq = max(128, -(-args.ctx[1] // B))
@@ -178,12 +194,19 @@ def bench_decode(args):
         PA.SPLIT_POLICY = "reference"
         st.seq_block_size, st.num_seq_blocks = args.force_split
 
+    def new_step():
+        # a serving loop builds its infer_state per step: what the wrappers keep on it (the balanced row
+        # order, one small launch) is recomputed in every timed step, inside the graph too
+        st.__dict__.pop("_morphkv_decode_order", None)
+
     def step_two_calls():
+        new_step()
         for layer in range(L):
             store_kvcache(k_new[layer], v_new[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer)
             paged_attention(q[layer], k_cache, v_cache, [], [], bt, model, engine, st, layer, o[layer])
 
     def step_fused():
+        new_step()
         for layer in range(L):
             decode_append_and_attend(k_new[layer], v_new[layer], q[layer], k_cache, v_cache, [], [], bt,
                                      model, engine, st, layer, o[layer])
@@ -323,7 +346,10 @@ def bench_decode(args):
                                + (", pool over HIP virtual memory" if args.pool_backing == "vmm" else ""),
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
-                   "timed_as": "eager launches" if graph is None else "HIP graph replay of one step"},
+                   "timed_as": "eager launches" if graph is None else "HIP graph replay of one step",
+                   "row_order": ("the grid takes the batch's rows in the balanced order, computed once per step "
+                                 "inside the timed region" if _balanced_order() else "the grid takes the rows as given")
+                                + (", lengths handed over pre-ordered (--seq-order snake)" if args.seq_order == "snake" else "")},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
         "us_per_step": round(ms_per_step * 1e3, 2),

@@ -157,6 +157,28 @@ int mkv_decode_rope_append_attn(const void* k, const void* v, const void* q,
                                 float softmax_scale, int32_t layer, int32_t tokens_per_split,
                                 int32_t max_splits, void* mid_o, void* mid_lse, void* stream);
 
+/* No counterpart in the reference (its kernels take the batch in the caller's order,
+ * MS/worker/kernels/paged_attn.py:59-77).  order[slot] = row of the decode batch that the
+ * workgroups at grid slot `slot` should take: the rows by descending length, dealt in snake order
+ * over runs of 256 / num_kv_heads slots, so that the workgroups sharing a CU stream about the same
+ * number of tokens.  It depends on seq_lens only: compute it once per batch and pass it to every
+ * layer's mkv_decode_attn_ordered.  n <= 4096. */
+int mkv_decode_order(const int32_t* seq_lens, int32_t n, int32_t num_kv_heads,
+                     int32_t* order, void* stream);
+
+/* mkv_paged_attn_decode / mkv_decode_append_attn / mkv_decode_rope_append_attn in one entry, with the
+ * order in which the grid takes the batch rows: order = NULL keeps the rows' own order (any
+ * permutation of 0..n-1 gives the same outputs); k, v = NULL: no append; cos_table, sin_table = NULL:
+ * no rotary (they need k, v).  Everything else as in the three entries above. */
+int mkv_decode_attn_ordered(const void* q, void* o, const mkv_pool* pool,
+                            const int32_t* block_table, int64_t max_blocks_per_seq,
+                            const int32_t* seq_ids, const int32_t* seq_lens,
+                            const int32_t* order, int32_t n, int32_t num_q_heads,
+                            float softmax_scale, int32_t layer, int32_t tokens_per_split,
+                            int32_t max_splits, void* mid_o, void* mid_lse,
+                            const void* k, const void* v, const void* cos_table,
+                            const void* sin_table, void* stream);
+
 /* ---- prefill attention -------------------------------------------------- */
 /* prefill_attention, MS/worker/kernels/prefill_attn.py:9-139, and the live
  * flash_attn_varlen_func call, MS/worker/layers/transformer_layer.py:154-164:

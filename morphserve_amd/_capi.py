@@ -53,6 +53,9 @@ PROTOTYPES = {
     "mkv_append_prefill": [_P, _P, _PP, _P, _I64, _P, _P, _P, _I32, _I32, _I32, _P],
     "mkv_paged_attn_scratch_bytes": [_I32, _I32, _I32, _I32, C.POINTER(_I64), C.POINTER(_I64)],
     "mkv_paged_attn_decode": [_P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32, _P, _P, _P],
+    "mkv_decode_order": [_P, _I32, _I32, _P, _P],
+    "mkv_decode_attn_ordered": [_P, _P, _PP, _P, _I64, _P, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32, _P, _P, _P, _P,
+                                _P, _P, _P],
     "mkv_paged_attn_decode_static": [_P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32, _P],
     "mkv_decode_append_attn": [_P, _P, _P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32, _P, _P, _P],
     "mkv_decode_rope_append_attn": [_P, _P, _P, _P, _P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32,

@@ -142,6 +142,33 @@ __device__ __forceinline__ void merge_waves_and_store(const float (&sm_acc)[4][G
     }
 }
 
+
+// Which sequence should the workgroup at batch slot w take?  With one split per sequence a launch holds
+// one workgroup per (kv head, sequence), and the CUs receive consecutive workgroups in turn: slots w
+// and w + 256 / Hkv end up on the same CU.  Dealing the sequences to the slots by length in snake
+// order (longest first over one run of 256 / Hkv slots, the next run reversed, ...) gives every CU
+// about the same number of tokens to stream, so a launch does not end on the CUs that happened to
+// draw two long sequences.  The order depends on the lengths only, so it is computed once per batch
+// (this kernel: one workgroup, rank by (length, row) with n compares per row) and handed to every
+// layer's launch.  order[slot] = row of the batch; any permutation is valid, this one is balanced.
+__global__ __launch_bounds__(1024) void decode_order_kernel(const int32_t* __restrict__ seq_lens, int32_t n,
+                                                            int32_t run, int32_t* __restrict__ order) {
+    __shared__ int32_t s_len[4096];
+    for (int j = threadIdx.x; j < n; j += blockDim.x) s_len[j] = seq_lens[j];
+    __syncthreads();
+    for (int j = threadIdx.x; j < n; j += blockDim.x) {
+        const int mine = s_len[j];
+        int rank = 0;                                   // rows that come before row j: longer, or as long and earlier
+        for (int k = 0; k < n; ++k) {
+            const int other = s_len[k];
+            rank += (other > mine) || (other == mine && k < j);
+        }
+        const int r = rank / run, c = rank - r * run;
+        const int slot = (r < n / run && (r & 1)) ? r * run + (run - 1 - c) : rank;    // a trailing partial run stays in order
+        order[slot] = j;
+    }
+}
+
 template <int G>
 __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ q,        // [n, Hq, D] fp16
@@ -154,14 +181,15 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ k_new,    // [n, Hkv, D] fp16 or NULL: token len-1 to append first
     const uint4* __restrict__ v_new,
     const uint4* __restrict__ cos_t,    // [n, D/2] fp16 or NULL: rotate q and the new k row on the way in
-    const uint4* __restrict__ sin_t) {
+    const uint4* __restrict__ sin_t,
+    const int32_t* __restrict__ order) {   // [n] or NULL: batch row taken by each slot of the grid
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int r = lane >> 4;       // token row within a group of four
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
-    const int i = blockIdx.z;
+    const int i = order ? order[blockIdx.z] : (int)blockIdx.z;
     const int Hq = pool.num_kv_heads * G;
 
     const int len = seq_lens[i];
@@ -378,7 +406,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ seq_lens, float scale2, int32_t layer, int32_t blocks_per_split,
     int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new,
-    const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t) {
+    const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t, const int32_t* __restrict__ order) {
     __shared__ __attribute__((aligned(16))) char stage[4][2][kLdsTile];
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
@@ -391,7 +419,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     const int c = lane >> 4;       // lane group
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
-    const int i = blockIdx.z;
+    const int i = order ? order[blockIdx.z] : (int)blockIdx.z;
     const int Hq = pool.num_kv_heads * G;
 
     const int len = seq_lens[i];
@@ -689,7 +717,7 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
                           int64_t max_blocks_per_seq, const int32_t* seq_ids,
                           const int32_t* seq_lens, float scale2, int32_t layer,
                           int32_t blocks_per_split, int32_t max_splits, const void* k_new,
-                          const void* v_new, const void* cos_t, const void* sin_t) {
+                          const void* v_new, const void* cos_t, const void* sin_t, const int32_t* order) {
     // the vector-ALU kernel exists for the power-of-two groups only; every other group
     // size (up to the 16 columns of a matrix tile) runs on the matrix cores
     constexpr bool has_valu = G == 1 || G == 2 || G == 4 || G == 8;
@@ -699,12 +727,13 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
                            (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
                            max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
                            max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
-                           (const uint4*)sin_t);
+                           (const uint4*)sin_t, order);
     } else if constexpr (has_valu) {
         hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
                            (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
                            seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
-                           (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t);
+                           (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t,
+                           order);
     }
 }
 
@@ -733,7 +762,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
                        int32_t n, int32_t num_q_heads, float softmax_scale, int32_t layer,
                        int32_t tokens_per_split, int32_t max_splits, void* mid_o, void* mid_lse,
                        const void* k_new, const void* v_new, const void* cos_t, const void* sin_t,
-                       void* stream) {
+                       void* stream, const int32_t* order = nullptr) {
     int rc = mkv::check_pool(pool);
     if (rc) return rc;
     MKV_REQUIRE(n >= 0, "n must be >= 0");
@@ -763,7 +792,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
     case GG:                                                                                       \
         mkv::launch_phase1<GG>(grid, s, q, o, mid_o, mid_lse, pool, block_table,                   \
                                max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, bps,          \
-                               max_splits, k_new, v_new, cos_t, sin_t);                            \
+                               max_splits, k_new, v_new, cos_t, sin_t, order);                     \
         break;
             MKV_CASE(1)
             MKV_CASE(2)
@@ -889,6 +918,37 @@ int mkv_decode_rope_append_attn(const void* k, const void* v, const void* q, con
     return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n,
                        num_q_heads, softmax_scale, layer, tokens_per_split, max_splits, mid_o,
                        mid_lse, k, v, cos_table, sin_table, stream);
+}
+
+int mkv_decode_order(const int32_t* seq_lens, int32_t n, int32_t num_kv_heads, int32_t* order, void* stream) {
+    MKV_REQUIRE(n >= 0, "n must be >= 0");
+    if (n == 0) return MKV_OK;
+    MKV_REQUIRE(seq_lens && order, "NULL argument");
+    MKV_REQUIRE(n <= 4096, "at most 4096 sequences (got %d)", n);
+    MKV_REQUIRE(num_kv_heads > 0, "num_kv_heads must be positive");
+    // slots one run apart share a CU (256 CUs, one workgroup per kv head and slot); when the kv heads do
+    // not divide the CU count there is no such pairing and the order is plain longest-first
+    const int run = (256 % num_kv_heads == 0 && 256 / num_kv_heads >= 1) ? 256 / num_kv_heads : n;
+    hipLaunchKernelGGL(mkv::decode_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seq_lens, n, run, order);
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
+
+int mkv_decode_attn_ordered(const void* q, void* o, const mkv_pool* pool, const int32_t* block_table,
+                            int64_t max_blocks_per_seq, const int32_t* seq_ids, const int32_t* seq_lens,
+                            const int32_t* order, int32_t n, int32_t num_q_heads, float softmax_scale,
+                            int32_t layer, int32_t tokens_per_split, int32_t max_splits, void* mid_o,
+                            void* mid_lse, const void* k, const void* v, const void* cos_table,
+                            const void* sin_table, void* stream) {
+    MKV_REQUIRE((k == nullptr) == (v == nullptr), "k and v go together");
+    MKV_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "cos and sin tables go together");
+    MKV_REQUIRE(!cos_table || k, "the rotary tables need the new k and v rows");
+    MKV_REQUIRE(((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0 && ((uintptr_t)cos_table & 15) == 0 &&
+                    ((uintptr_t)sin_table & 15) == 0 && ((uintptr_t)order & 3) == 0,
+                "k/v/cos/sin must be 16-byte aligned, order 4-byte aligned");
+    return decode_impl(q, o, pool, block_table, max_blocks_per_seq, seq_ids, seq_lens, n, num_q_heads,
+                       softmax_scale, layer, tokens_per_split, max_splits, mid_o, mid_lse, k, v, cos_table,
+                       sin_table, stream, order);
 }
 
 }  // extern "C"

@@ -24,6 +24,9 @@ _scratch: Dict[Tuple[int, int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
 # caller's infer_state.seq_block_size as the reference kernels do.
 SPLIT_POLICY = os.environ.get("MORPHKV_SPLIT_POLICY", "auto")
 TARGET_WORKGROUPS = int(os.environ.get("MORPHKV_TARGET_WGS", "512"))
+# The grid takes the batch rows in an order that gives every CU about the same number of tokens
+# (``mkv_decode_order``); "0" keeps the rows' own order.
+BALANCED_ORDER = os.environ.get("MORPHKV_DECODE_ORDER", "1") != "0"
 
 
 def choose_split(n: int, num_kv_heads: int, max_len: int, block_size: int,
@@ -54,6 +57,34 @@ def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
                torch.empty(grow, dtype=torch.float32, device=device))
         _scratch[key] = cur
     return cur
+
+
+def _decode_order(infer_state, lens: torch.Tensor, n: int, num_kv_heads: int) -> Optional[torch.Tensor]:
+    """The balanced order of this batch's rows, computed by one small launch the first time a layer asks
+    for it and kept on ``infer_state`` for the other layers of the step (it depends on the lengths only).
+    An order that has gone stale -- lengths updated in place -- is still a permutation, so the outputs
+    do not depend on it; only the balance does."""
+    if not BALANCED_ORDER or n < 2 or n > 4096:
+        return None
+    key = (lens.data_ptr(), n, num_kv_heads)
+    cached = getattr(infer_state, "_morphkv_decode_order", None)
+    stream = torch.cuda.current_stream()
+    capturing = torch.cuda.is_current_stream_capturing()
+    if cached is None or cached[0] != key:
+        order = torch.empty(n, dtype=torch.int32, device=lens.device)
+        cached = [key, order, None, stream.cuda_stream]
+        try:
+            infer_state._morphkv_decode_order = cached
+        except AttributeError:          # nowhere to keep it: a launch per layer would cost more than it brings
+            return None
+        _capi.check(_capi.lib().mkv_decode_order(lens.data_ptr(), n, num_kv_heads, order.data_ptr(),
+                                                 stream.cuda_stream))
+        if not capturing:
+            cached[2] = torch.cuda.Event()
+            cached[2].record(stream)
+    elif cached[3] != stream.cuda_stream and cached[2] is not None and not capturing:
+        stream.wait_event(cached[2])    # computed on another stream
+    return cached[1]
 
 
 def _split_for(infer_state, model_config, engine_config):
@@ -101,11 +132,12 @@ def decode_append_and_attend(
     mid_o, mid_lse = (None, None)
     if splits > 1:
         mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
-    _capi.check(_capi.lib().mkv_decode_append_attn(
-        k.data_ptr(), v.data_ptr(), q.data_ptr(), o.data_ptr(), C.byref(pool),
-        block_table.data_ptr(), block_table.shape[1], infer_state.seq_ids.data_ptr(),
-        infer_state.decoding_seq_lens.data_ptr(), n, hq, float(infer_state.softmax_scale),
-        cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    _capi.check(_capi.lib().mkv_decode_attn_ordered(
+        q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
+        infer_state.seq_ids.data_ptr(), infer_state.decoding_seq_lens.data_ptr(), _capi.ptr(order), n, hq,
+        float(infer_state.softmax_scale), cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse),
+        k.data_ptr(), v.data_ptr(), None, None, _capi.current_stream()))
 
 
 def decode_rope_append_and_attend(
@@ -144,11 +176,12 @@ def decode_rope_append_and_attend(
     mid_o, mid_lse = (None, None)
     if splits > 1:
         mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
-    _capi.check(_capi.lib().mkv_decode_rope_append_attn(
-        k.data_ptr(), v.data_ptr(), q.data_ptr(), cos.data_ptr(), sin.data_ptr(), o.data_ptr(), C.byref(pool),
-        block_table.data_ptr(), block_table.shape[1], infer_state.seq_ids.data_ptr(),
-        infer_state.decoding_seq_lens.data_ptr(), n, hq, float(infer_state.softmax_scale),
-        cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    _capi.check(_capi.lib().mkv_decode_attn_ordered(
+        q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
+        infer_state.seq_ids.data_ptr(), infer_state.decoding_seq_lens.data_ptr(), _capi.ptr(order), n, hq,
+        float(infer_state.softmax_scale), cur_layer, tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse),
+        k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(), _capi.current_stream()))
 
 
 def paged_attention(
@@ -190,15 +223,10 @@ def paged_attention(
     seq_ids_ptr = infer_state.seq_ids.data_ptr() + ids_off
     lens_ptr = infer_state.decoding_seq_lens.data_ptr()
     pending = _deferred.take(k_cache, v_cache, block_table, seq_ids_ptr, lens_ptr, n, cur_layer)
-    if pending is not None:
-        # the decode rows store_kvcache was given for this layer are appended by this launch
-        _capi.check(lib.mkv_decode_append_attn(
-            pending.k_ptr, pending.v_ptr, q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(),
-            block_table.shape[1], seq_ids_ptr, lens_ptr, n, hq, float(infer_state.softmax_scale), cur_layer,
-            tps, splits, _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
-        return
-    _capi.check(lib.mkv_paged_attn_decode(
-        q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
-        seq_ids_ptr, lens_ptr,
-        n, hq, float(infer_state.softmax_scale), cur_layer, tps, splits,
-        _capi.ptr(mid_o), _capi.ptr(mid_lse), _capi.current_stream()))
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    # a pending append: the decode rows store_kvcache was given for this layer are appended by this launch
+    _capi.check(lib.mkv_decode_attn_ordered(
+        q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1], seq_ids_ptr,
+        lens_ptr, _capi.ptr(order), n, hq, float(infer_state.softmax_scale), cur_layer, tps, splits,
+        _capi.ptr(mid_o), _capi.ptr(mid_lse), pending.k_ptr if pending is not None else None,
+        pending.v_ptr if pending is not None else None, None, None, _capi.current_stream()))

@@ -33,6 +33,7 @@ def test_the_reference_facing_header_holds_no_tuning_or_measurement_entries():
 def test_header_declares_the_expected_surface():
     names = _declared()
     for must in ("mkv_append_decode", "mkv_append_prefill", "mkv_paged_attn_decode", "mkv_prefill_attn",
+                 "mkv_decode_order", "mkv_decode_attn_ordered",
                  "mkv_bm_allocate", "mkv_bt_append", "mkv_bt_release", "mkv_bt_gather_release",
                  "mkv_pool_plan_shrink", "mkv_pool_migrate", "mkv_bt_remap", "mkv_swap_blocks",
                  "mkv_pool_carve_segment", "mkv_fill_zero"):
@@ -159,6 +160,13 @@ def test_bad_arguments_are_refused_before_any_launch():
         "mkv_paged_attn_decode_static/too large": (A, A, G, A, 4, A, A, 64, 64, 0.1, 0, 64, 64, None),
         "mkv_decode_append_attn": (A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
         "mkv_decode_rope_append_attn": (A, A, A, A, A, A, P, A, 4, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None),
+        "mkv_decode_order": (None, 4, 8, A, None),
+        "mkv_decode_order/too many rows": (A, 4097, 8, A, None),
+        "mkv_decode_order/heads": (A, 4, 0, A, None),
+        "mkv_decode_attn_ordered": (A, A, P, A, 4, A, A, A, 1, 2, 0.1, 0, 64, 1, None, None, None, None, None, None,
+                                    None),
+        "mkv_decode_attn_ordered/k without v": (A, A, G, A, 4, A, A, None, 1, 2, 0.1, 0, 64, 1, None, None, A, None,
+                                                None, None, None),
         "mkv_prefill_attn": (A, A, A, A, A, A, 1, 16, 2, 2, 64, 0.1, None),                  # head_dim 64
         "mkv_prefill_attn/scale": (A, A, A, A, A, A, 1, 16, 2, 2, 128, 0.0, None),
         "mkv_prefill_attn_paged": (A, A, P, A, 4, A, A, A, None, 1, 16, 2, 0.1, 0, None),
