@@ -183,7 +183,7 @@ int mkv_decode_attn_ordered(const void* q, void* o, const mkv_pool* pool,
 /* prefill_attention, MS/worker/kernels/prefill_attn.py:9-139, and the live
  * flash_attn_varlen_func call, MS/worker/layers/transformer_layer.py:154-164:
  * causal attention of each prefill sequence over its own contiguous q, k, v.
- * q, o : [T, Hq, D] fp16; k, v : [T, Hkv, D] fp16. */
+ * q, o : [T, Hq, D] fp16; k, v : [T, Hkv, D] fp16; all four 16-byte aligned. */
 int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
                      const int32_t* start_locs, const int32_t* seq_lens,
                      int32_t num_seqs, int32_t max_len, int32_t num_q_heads,
@@ -195,7 +195,8 @@ int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
  * MS/worker/layers/transformer_layer.py:151-164).  Chunk b holds chunk_lens[b]
  * query rows at positions prefix_lens[b] .. of sequence seq_ids[b]; K/V of every
  * position up to the chunk's end are already in the cache (append first); row at
- * position p attends to cached positions <= p.  prefix_lens may be NULL (= 0). */
+ * position p attends to cached positions <= p.  prefix_lens may be NULL (= 0).
+ * q and o 16-byte aligned. */
 int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
                            const int32_t* block_table, int64_t max_blocks_per_seq,
                            const int32_t* seq_ids, const int32_t* start_locs,

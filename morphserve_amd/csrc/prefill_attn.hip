@@ -17,6 +17,10 @@
 // running max is reduced over the four lane groups that share it with the
 // lane-swap instructions.  Tiles entirely below a wave's diagonal take a body
 // without any masking; only the one or two diagonal tiles pay for the compares.
+// The output leaves through LDS: each wave transposes its column tiles in a corner
+// of the idle V buffer and writes whole 256-byte rows, 16 bytes per lane.  In the
+// four-wave shape a workgroup that carries two query tiles requests the second
+// tile's q and first K/V tile while the first tile's last key tile is consumed.
 //
 // Two K/V sources: the batch's own contiguous k, v ([T, Hkv, D]) -- the
 // reference's whole-prompt prefill -- or the paged cache through the block
@@ -142,11 +146,23 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int64_t start = a.start_locs[b];
     const int prefix = (PAGED && a.prefix_lens) ? a.prefix_lens[b] : 0;
 
+  // State that outlives a part: while the last key tile of part 0 is consumed, q and the first K/V
+  // tile(s) of part 1 are already requested, so the second part starts without a trip to memory.
+  constexpr int kFetchStepsO = (kKTile * 16) / (64 * WAVES);
+  v8h qb[kU][4];
+  v4u kreg[WAVES == 8 ? 2 : 1][kFetchStepsO], vreg[WAVES == 8 ? 2 : 1][kFetchStepsO];
+  int32_t tile_ids = 0;
+  int f_kv_len = 0;                   // the fetch side's view: keys of the part whose tiles are being requested
+  uint32_t last_off = 0, next_off = 0;
+  bool carried = false;               // this part's q and first tile(s) were requested by the previous part
   for (int part = 0; part < 2; ++part) {
     const int qt = part == 0 ? n_qt - 1 - ti : ti;
     if (part == 1 && (!a.pair_tiles || 2 * ti == n_qt - 1)) break;   // unpaired, or odd count: the middle tile was part 0
     const int q0 = qt * kQTile;
     const int kv_len = prefix + min(len, q0 + kQTile);       // keys this workgroup can see
+    const bool more = WAVES == 4 && part == 0 && a.pair_tiles && 2 * ti != n_qt - 1;   // a second part follows (short-prompt shape only)
+    const int nx_q0 = ti * kQTile;
+    int nx_kv_len = more ? prefix + min(len, nx_q0 + kQTile) : 0;
 
     // this wave's 32 rows: chunk-local rows r0w .. r0w+31, column tile u = rows r0w+16u ..
     const int r0w = q0 + wave * (16 * kU);
@@ -161,18 +177,22 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 
     // Q^T as B operand: lane (row m, group c) holds dims c*32 + 8x .. +8 for product x
     // (the contraction order over dims is free; K uses the same order).
-    v8h qb[kU][4];
+    auto load_q = [&](int tile_q0) {
+        if (WAVES == 4) asm volatile("" : "+s"(tile_q0));      // the addresses are formed here, not ahead of the tile loop
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-        if (my_row[u] < len) {
-            const uint4* qp = (const uint4*)(a.q + ((start + my_row[u]) * Hq + hq) * kPD + c * 32);
+        for (int u = 0; u < kU; ++u) {
+            const int row = tile_q0 + wave * (16 * kU) + u * 16 + m;
+            if (row < len) {
+                const uint4* qp = (const uint4*)(a.q + ((start + row) * Hq + hq) * kPD + c * 32);
 #pragma unroll
-            for (int x = 0; x < 4; ++x) qb[u][x] = __builtin_bit_cast(v8h, qp[x]);
-        } else {
+                for (int x = 0; x < 4; ++x) qb[u][x] = __builtin_bit_cast(v8h, qp[x]);
+            } else {
 #pragma unroll
-            for (int x = 0; x < 4; ++x) qb[u][x] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
+                for (int x = 0; x < 4; ++x) qb[u][x] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
+            }
         }
-    }
+    };
+    if (!carried) load_q(q0);
 
     v4f acc[kU][8];                    // O^T tiles: dims 16t + 4c + j, query row m of column tile u
 #pragma unroll
@@ -200,24 +220,29 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     // probabilities are zero); unmapped table entries read as zeros.
     // Contiguous source: one uniform base per (sequence, kv head) plus a 32-bit byte offset
     // per lane that advances by a constant per tile (the launcher bounds len * Hkv * 256).
-    v4u kreg[kSets][kFetchSteps], vreg[kSets][kFetchSteps];
+    static_assert(kFetchSteps == kFetchStepsO, "staging register count");
     const uint32_t row_stride = (uint32_t)Hkv * (kPD * 2);
     const char* k_src = PAGED ? nullptr : (const char*)a.k + (start * Hkv + kvh) * (int64_t)(kPD * 2);
     const char* v_src = PAGED ? nullptr : (const char*)a.v + (start * Hkv + kvh) * (int64_t)(kPD * 2);
-    const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + (tid & 15) * 16;
-    uint32_t next_off = (uint32_t)(tid >> 4) * row_stride + (tid & 15) * 16;     // key (tid >> 4) of the next tile
+    auto begin_fetch = [&](int kvl) {
+        f_kv_len = kvl;
+        last_off = (uint32_t)(kvl - 1) * row_stride + (tid & 15) * 16;
+        next_off = (uint32_t)(tid >> 4) * row_stride + (tid & 15) * 16;          // key (tid >> 4) of the next tile
+    };
     // Paged source: fetch step u covers keys key0 + 16u .. +15 = ONE block (block_size is 16
     // here), so its id and address are workgroup-uniform and only the row inside it differs
     // per thread.  The four ids of a tile are loaded one tile ahead (lane u keeps step u's),
     // so no fetch ever waits on a table lookup.
-    int32_t tile_ids = 0;
-    auto load_tile_ids = [&](int key0) {
+    auto load_tile_ids = [&](int key0, int kvl) {
         if (PAGED) {      // entries past the table row name no block: they read as zeros, never as a neighbour's row
-            const int idx = min((key0 >> 4) + (lane & 3), (kv_len - 1) >> 4);
+            const int idx = min((key0 >> 4) + (lane & 3), (kvl - 1) >> 4);
             tile_ids = idx < a.max_blocks_per_seq ? bt_row[idx] : -1;
         }
     };
-    load_tile_ids(0);
+    if (!carried) {
+        begin_fetch(kv_len);
+        load_tile_ids(0, kv_len);
+    }
     auto fetch_tile = [&](int key0, auto set_tag) {
         constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
@@ -225,8 +250,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             if (PAGED) {
                 // a step covers kStepRows keys = kStepRows / 16 blocks; a wave's rows lie in one of them
                 const int blk_in_tile = (kStepRows / 16) * u + ((tid >> 4) >> 4);      // wave-uniform
-                const int blk = min((key0 >> 4) + blk_in_tile, (kv_len - 1) >> 4);
-                const int pos = min(key0 + kStepRows * u + (tid >> 4), kv_len - 1);
+                const int blk = min((key0 >> 4) + blk_in_tile, (f_kv_len - 1) >> 4);
+                const int pos = min(key0 + kStepRows * u + (tid >> 4), f_kv_len - 1);
                 const int64_t pid = __builtin_amdgcn_readlane(tile_ids, __builtin_amdgcn_readfirstlane(blk_in_tile));
                 kreg[SET][u] = (v4u){0u, 0u, 0u, 0u};
                 vreg[SET][u] = kreg[SET][u];
@@ -244,7 +269,12 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         }
         next_off += kKTile * row_stride;
-        load_tile_ids(key0 + kKTile);
+        // the ids of the tile after this one; after a part's last tile, those of the next part's first
+        if (nx_kv_len != 0 && key0 + kKTile >= f_kv_len) {
+            load_tile_ids(0, nx_kv_len);
+        } else {
+            load_tile_ids(key0 + kKTile, f_kv_len);
+        }
     };
     const int k_wr_off = (tid >> 4) * kRowBytes + (tid & 15) * 16;           // + 16u rows
     const int v_wr_off = (tid >> 4) * kRowBytesV + (tid & 15) * 16;
@@ -263,7 +293,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int v_rd_off = (4 * c + (m >> 2)) * kRowBytesV + (m & 3) * 8;     // + 16n rows, + 32t bytes
 
     // one 64-key tile against this wave's 32 rows
-    auto tile_body = [&](auto masked_tag, int buf, int key0, const uint4 (&kf_first)[4]) {
+    auto tile_body = [&](auto masked_tag, int buf, int key0, const uint4 (&kf_first)[4], int reload_q0) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         const char* k_rd = k_lds + buf * kKBuf + k_rd_off;
         const char* v_rd = v_lds + buf * kVBuf + v_rd_off;
@@ -317,6 +347,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             va_pre[t] = __builtin_bit_cast(v8h, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
         __builtin_amdgcn_sched_barrier(0);
+        // the scores were q's last use in this part: the next part's q is requested here
+        if (reload_q0 >= 0) load_q(reload_q0);
         // ---- online softmax per column tile -----------------------------------------------
         __builtin_amdgcn_s_setprio(0);
         v8h pb[kU][2];                 // P^T as B operand: [pair of sub-tiles] = 8 k-slots
@@ -407,18 +439,21 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         }
         if (active) {
             if (key0 + kKTile - 1 <= wave_min_pos) {  // every row sees every key (and all keys < kv_len)
-                tile_body(std::false_type{}, buf, key0, kf_first);
+                tile_body(std::false_type{}, buf, key0, kf_first, -1);
             } else {
-                tile_body(std::true_type{}, buf, key0, kf_first);
+                tile_body(std::true_type{}, buf, key0, kf_first, -1);
             }
         }
         stage_tile(buf ^ 1, nxt_set);                 // the other buffer: last read one iteration ago
         __syncthreads();
     };
-    fetch_tile(0, Set0{});
-    if (kSets == 2 && num_tiles > 1) fetch_tile(kKTile, Set1{});
-    stage_tile(0, Set0{});
-    __syncthreads();
+    if (!carried) {
+        fetch_tile(0, Set0{});
+        if (kSets == 2 && num_tiles > 1) fetch_tile(kKTile, Set1{});
+        stage_tile(0, Set0{});
+        __syncthreads();
+    }
+    carried = false;
     for (int it = 0; it + 1 < num_tiles; it += 2) {
         iteration(it, Set0{}, Set1{});
         if (it + 2 < num_tiles) iteration(it + 1, Set1{}, Set0{});
@@ -426,27 +461,54 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     {   // the last tile holds the workgroup's diagonal: never fully visible to a wave
         const int it = num_tiles - 1;
         const int key0 = it * kKTile;
-        if (wave_has_rows && key0 <= wave_max_pos) {
-            uint4 kf_first[4];
-            first_frags(it & 1, kf_first);
-            tile_body(std::true_type{}, it & 1, key0, kf_first);
+        const bool active = wave_has_rows && key0 <= wave_max_pos;
+        uint4 kf_first[4];
+        if (active) first_frags(it & 1, kf_first);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) {                                   // both staging sets are idle: the next part's first tile(s)
+            int kvl = nx_kv_len;
+            asm volatile("" : "+s"(kvl));             // keeps the next part's addresses out of the tile loop's registers
+            const int nx_tiles = (kvl + kKTile - 1) / kKTile;
+            begin_fetch(kvl);
+            nx_kv_len = 0;
+            fetch_tile(0, Set0{});
+            if (kSets == 2 && nx_tiles > 1) fetch_tile(kKTile, Set1{});
         }
-        __syncthreads();                              // the next part restages buffer 0
+        if (active) {
+            tile_body(std::true_type{}, it & 1, key0, kf_first, more ? nx_q0 : -1);
+        } else if (more) {
+            load_q(nx_q0);
+        }
+        __syncthreads();                              // every read of the staged tiles is done
     }
 
+    // Output: a lane holds four dims of sixteen rows' worth of 8-byte pieces; the column tile goes
+    // through this wave's corner of the idle V buffer (rows 288 bytes apart: conflict-free 8-byte
+    // writes) and comes back as whole rows, so that o is written 256 contiguous bytes per row,
+    // 16 bytes per lane.  The four-wave shape keeps V buffer 0 for the next part's first tile.
+    {
+        constexpr int kORow = 288;
+        char* o_lds = v_lds + (WAVES == 4 ? kVBuf : 0) + wave * (16 * kORow);
+        const bool follows = part == 0 && a.pair_tiles && 2 * ti != n_qt - 1;
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-        const float l_tot = lsum[u][0];
-        if (my_row[u] < len) {
-            const float inv = 1.f / l_tot;
-            __half* op = a.o + ((start + my_row[u]) * Hq + hq) * kPD;
+        for (int u = 0; u < kU; ++u) {
+            const float inv = 1.f / lsum[u][0];
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const v4h out = (v4h){(_Float16)(acc[u][t][0] * inv), (_Float16)(acc[u][t][1] * inv),
                                       (_Float16)(acc[u][t][2] * inv), (_Float16)(acc[u][t][3] * inv)};
-                *(uint2*)(op + 16 * t + 4 * c) = __builtin_bit_cast(uint2, out);
+                *(uint2*)(o_lds + m * kORow + 32 * t + 8 * c) = __builtin_bit_cast(uint2, out);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 orow = *(const uint4*)(o_lds + (4 * i + c) * kORow + 16 * m);
+                const int row = r0w + u * 16 + 4 * i + c;
+                if (row < len) *(uint4*)(a.o + ((start + row) * Hq + hq) * kPD + 8 * m) = orow;
             }
         }
+        if (more) stage_tile(0, Set0{});
+        if (follows) __syncthreads();                 // the next part's staging may reuse every buffer
+        if (more) carried = true;
     }
   }   // part
 }
@@ -518,8 +580,8 @@ int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
     MKV_REQUIRE(softmax_scale > 0.f, "softmax_scale must be positive");
     MKV_REQUIRE((int64_t)max_len * num_kv_heads < (1 << 23), "max_len * num_kv_heads must be below 2^23");
     MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)k & 15) == 0 && ((uintptr_t)v & 15) == 0 &&
-                    ((uintptr_t)o & 7) == 0,
-                "q/k/v must be 16-byte aligned, o 8-byte aligned");
+                    ((uintptr_t)o & 15) == 0,
+                "q/k/v/o must be 16-byte aligned");
     mkv::PrefillArgs a = {};
     a.q = (const __half*)q;
     a.o = (__half*)o;
@@ -551,8 +613,8 @@ int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
                 "num_q_heads %d must be a multiple of num_kv_heads %d", num_q_heads, pool->num_kv_heads);
     MKV_REQUIRE(num_seqs <= 65535 && num_q_heads <= 65535, "grid dimension limit");
     MKV_REQUIRE(softmax_scale > 0.f, "softmax_scale must be positive");
-    MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)o & 7) == 0,
-                "q must be 16-byte aligned, o 8-byte aligned");
+    MKV_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)o & 15) == 0,
+                "q and o must be 16-byte aligned");
     mkv::PrefillArgs a = {};
     a.q = (const __half*)q;
     a.o = (__half*)o;
