@@ -83,7 +83,8 @@ def parse_args():
     ap.add_argument("--force-split", type=int, nargs=2, default=None, metavar=("TOKENS", "SPLITS"),
                     help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
-                    help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches")
+                    help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches; SEQSxTOKENS+PREFIX is a "
+                         "batch of chunks over PREFIX tokens already in a paged cache")
     ap.add_argument("--seq-order", choices=["drawn", "snake"], default="drawn",
                     help="decode workloads, diagnostic: keep the drawn order of context lengths, or hand the batch over "
                          "sorted so that slots 256 / Hkv apart (the two workgroups of a CU) hold a long and a short one")
@@ -1035,9 +1036,10 @@ def bench_mfma_calibration(args):
 
 
 def bench_prefill_shapes(args):
-    """Causal prefill attention over the batch's own contiguous q, k, v (MHA 32 / 32 heads, head_dim 128) for
-    a list of prompt batches and every workgroup shape of the kernel: microseconds per launch and TFLOP/s
-    (causal half, QK^T + PV).  `value` is the library's own choice on the first shape."""
+    """Causal prefill attention (MHA 32 / 32 heads, head_dim 128) for a list of prompt batches -- whole prompts
+    over the batch's own contiguous q, k, v ("8x512"), or chunks over a prefix already in a paged cache
+    ("8x512+2048") -- and every workgroup shape of the kernel: microseconds per launch and TFLOP/s (causal
+    half of the chunk plus the whole prefix, QK^T + PV).  `value` is the library's own choice on the first shape."""
     import torch
     from morphserve_amd import _capi
 
@@ -1049,7 +1051,12 @@ def bench_prefill_shapes(args):
     variants = [int(x) for x in args.prefill_variants.split(",")]
     rows = {}
     for shape in args.prefill_shapes.split(","):
-        nseq, ln = (int(x) for x in shape.split("x"))
+        # "NxL": N whole prompts of L tokens over their own k, v; "NxL+P": N chunks of L tokens whose sequences
+        # already hold P tokens in a paged cache (one layer, blocks dealt from a seeded permutation of the pool)
+        body, _, pfx = shape.partition("+")
+        prefix = int(pfx) if pfx else 0
+        paged = pfx != ""
+        nseq, ln = (int(x) for x in body.split("x"))
         T = nseq * ln
         if args.prefill_data == "zeros":
             q, k, v = (torch.zeros((T, H, D), dtype=torch.float16, device=dev) for _ in range(3))
@@ -1059,15 +1066,36 @@ def bench_prefill_shapes(args):
             v = torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g)
         starts = torch.arange(nseq, dtype=torch.int32, device=dev) * ln
         lens = torch.full((nseq,), ln, dtype=torch.int32, device=dev)
-        flops = nseq * H * 4 * D * ln * ln / 2
+        flops = nseq * H * 4 * D * (ln * prefix + ln * ln / 2)
+        if paged:
+            from morphserve_amd import build_infer_state, chunked_prefill_attention
+            per_seq = (prefix + ln + 15) // 16
+            nb = nseq * per_seq + 64
+            rng = np.random.default_rng(args.seed)
+            table = rng.permutation(nb)[:nseq * per_seq].reshape(nseq, per_seq).astype(np.int32)
+            bt = torch.from_numpy(table).to(dev)
+            if args.prefill_data == "zeros":
+                k_cache = torch.zeros((nb, 1, H, 16, D), dtype=torch.float16, device=dev)
+                v_cache = torch.zeros((nb, 1, H, 16, D), dtype=torch.float16, device=dev)
+            else:
+                k_cache = torch.randn((nb, 1, H, 16, D), dtype=torch.float16, device=dev, generator=g)
+                v_cache = torch.randn((nb, 1, H, 16, D), dtype=torch.float16, device=dev, generator=g)
+            model = Cfg(num_layers=1, num_q_heads=H, num_kv_heads=H, head_dim=D)
+            engine = Cfg(block_size=16, max_blocks_per_seq=per_seq)
+            st = build_infer_state([ln] * nseq, list(range(nseq)), [], H, D)
+            prefix_t = torch.full((nseq,), prefix, dtype=torch.int32, device=dev)
         outs, row = {}, {}
         for var in variants:
             _capi.check(lib.mkv_set_prefill_variant(var))
             o = torch.full_like(q, float("nan"))
 
             def run():
-                _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), starts.data_ptr(),
-                                                 lens.data_ptr(), nseq, ln, H, H, D, D ** -0.5, _capi.current_stream()))
+                if paged:
+                    chunked_prefill_attention(q, k_cache, v_cache, [], [], bt, model, engine, st, 0, o, prefix_t, prefix)
+                else:
+                    _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                     starts.data_ptr(), lens.data_ptr(), nseq, ln, H, H, D, D ** -0.5,
+                                                     _capi.current_stream()))
             # warm up by time, not by count: after the set-up kernels (random fills) the first few tens of
             # milliseconds of matrix work run at another clock, and a timing taken there reads 10-15 % low
             t_warm = time.perf_counter()

@@ -196,13 +196,14 @@ int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
  * query rows at positions prefix_lens[b] .. of sequence seq_ids[b]; K/V of every
  * position up to the chunk's end are already in the cache (append first); row at
  * position p attends to cached positions <= p.  prefix_lens may be NULL (= 0).
- * q and o 16-byte aligned. */
+ * max_prefix_len is a host-side upper bound of prefix_lens used only to choose the
+ * launch shape (0 = unknown; results do not depend on it).  q and o 16-byte aligned. */
 int mkv_prefill_attn_paged(const void* q, void* o, const mkv_pool* pool,
                            const int32_t* block_table, int64_t max_blocks_per_seq,
                            const int32_t* seq_ids, const int32_t* start_locs,
                            const int32_t* chunk_lens, const int32_t* prefix_lens,
-                           int32_t num_seqs, int32_t max_chunk_len, int32_t num_q_heads,
-                           float softmax_scale, int32_t layer, void* stream);
+                           int32_t num_seqs, int32_t max_chunk_len, int32_t max_prefix_len,
+                           int32_t num_q_heads, float softmax_scale, int32_t layer, void* stream);
 
 /* ---- block manager ------------------------------------------------------ */
 /* BlockManager.allocate_blocks_for_seqs, MS/worker/block_manager.py:64-112 with

@@ -63,7 +63,7 @@ PROTOTYPES = {
     "mkv_set_decode_variant": [_I32],
     "mkv_set_prefill_variant": [_I32],
     "mkv_prefill_attn": [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _F32, _P],
-    "mkv_prefill_attn_paged": [_P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _F32, _I32, _P],
+    "mkv_prefill_attn_paged": [_P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F32, _I32, _P],
     "mkv_bm_allocate": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I32, _I32, _P, _I64, _P, _P],
     "mkv_bm_take_first_free": [_P, _I64, _I64, _P, _P, _P],
     "mkv_bt_append": [_P, _I64, _P, _I64, _P, _P, _P, _I32, _I32, _P],

@@ -53,6 +53,7 @@ def chunked_prefill_attention(
     cur_layer: int,
     o: torch.Tensor,                    # [num_chunk_tokens, num_q_heads, head_dim], written
     prefix_lens: Optional[torch.Tensor] = None,   # [num_prefill_seqs] int32 cached tokens before each chunk
+    max_prefix_len: int = 0,            # host-side upper bound of prefix_lens (0 = unknown): picks the launch shape only
 ) -> None:
     """Chunk b = rows ``prefill_seq_start_locs[b] : +prefill_seq_lens[b]`` of ``q``
     at positions ``prefix_lens[b] ..`` of sequence ``seq_ids[b]``.  The chunk's own
@@ -68,5 +69,5 @@ def chunked_prefill_attention(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
         infer_state.seq_ids.data_ptr(), infer_state.prefill_seq_start_locs.data_ptr(),
         infer_state.prefill_seq_lens.data_ptr(), _capi.ptr(prefix_lens),
-        infer_state.num_prefill_seqs, infer_state.max_prefill_len, model_config.num_q_heads,
+        infer_state.num_prefill_seqs, infer_state.max_prefill_len, int(max_prefix_len), model_config.num_q_heads,
         float(infer_state.softmax_scale), cur_layer, _capi.current_stream()))

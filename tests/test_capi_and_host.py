@@ -169,7 +169,7 @@ def test_bad_arguments_are_refused_before_any_launch():
                                                 None, None, None),
         "mkv_prefill_attn": (A, A, A, A, A, A, 1, 16, 2, 2, 64, 0.1, None),                  # head_dim 64
         "mkv_prefill_attn/scale": (A, A, A, A, A, A, 1, 16, 2, 2, 128, 0.0, None),
-        "mkv_prefill_attn_paged": (A, A, P, A, 4, A, A, A, None, 1, 16, 2, 0.1, 0, None),
+        "mkv_prefill_attn_paged": (A, A, P, A, 4, A, A, A, None, 1, 16, 0, 2, 0.1, 0, None),
         "mkv_pool_migrate": (P, A, A, 1, None),
         "mkv_fill_zero": (A + 4, 64, None),                                                    # unaligned
         "mkv_swap_blocks": (None, None, 1, 0, P, None, None, None, None),

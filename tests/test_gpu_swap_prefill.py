@@ -157,6 +157,40 @@ def test_prefill_attention_both_workgroup_shapes(cuda, waves):
     assert_attn_close(o2.cpu().numpy(), want2, f"chunk over prefix, {waves} waves")
 
 
+def test_chunk_over_long_prefix_with_the_prefix_hint(cuda):
+    """Eight chunks over long cached prefixes, a grid wide enough for the library to pick the 256-row workgroup
+    shape when it is told how long the prefixes are: the hint must not change a bit, and both match the oracle."""
+    rng = np.random.default_rng(505)
+    Hq, Hkv = 32, 8
+    prefix = np.array([768, 600, 512, 1000, 530, 777, 640, 901])
+    chunk = np.array([256, 300, 512, 257, 384, 256, 400, 333])
+    lens = prefix + chunk
+    T = int(lens.sum())
+    k = rand_f16(rng, T, Hkv, 128)
+    v = rand_f16(rng, T, Hkv, 128)
+    starts = np.cumsum(lens) - lens
+    case = make_case(505, 1, Hq, Hkv, lens, num_blocks=int(((lens + 15) // 16).sum()) + 3, fill="all")
+    kc, vc, bt = to_gpu(case, cuda)
+    model, engine = configs(case)
+    st = build_infer_state(lens.tolist(), case.seq_ids.tolist(), [], Hkv, 128)
+    store_kvcache(torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda), kc, vc, [], [], bt, model, engine, st, 0)
+    R.append_prefill(case.arena, case.lay, k, v, case.block_table, case.seq_ids, starts, lens, 0)
+    s2 = np.cumsum(chunk) - chunk
+    q2 = rand_f16(rng, int(chunk.sum()), Hq, 128)
+    want = R.chunked_prefill_attention(q2, case.arena, case.lay, case.block_table, case.seq_ids, s2, chunk, prefix,
+                                       128 ** -0.5, 0)
+    st2 = build_infer_state(chunk.tolist(), case.seq_ids.tolist(), [], Hkv, 128)
+    outs = []
+    for hint in (0, int(prefix.max())):
+        o = torch.full((int(chunk.sum()), Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
+        chunked_prefill_attention(torch.from_numpy(q2).to(cuda), kc, vc, [], [], bt, model, engine, st2, 0, o,
+                                  prefix_lens=torch.from_numpy(prefix.astype(np.int32)).to(cuda), max_prefix_len=hint)
+        torch.cuda.synchronize()
+        outs.append(o.cpu().numpy())
+    assert_attn_close(outs[0], want, "chunk over long prefix, no hint")
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16)), "the prefix hint changed the output"
+
+
 def test_chunked_prefill_over_paged_cache(cuda):
     """Second half of each prompt as a chunk whose first half is already cached."""
     rng = np.random.default_rng(77)
