@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes", "placement_probe"])
+                             "eviction", "prefill_shapes", "placement_probe", "timeline"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -85,6 +85,8 @@ def parse_args():
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches; SEQSxTOKENS+PREFIX is a "
                          "batch of chunks over PREFIX tokens already in a paged cache")
+    ap.add_argument("--timeline-decode", default="64x1024-1536,1x32768,16x2048",
+                    help="timeline workload: comma-separated BATCHxLO-HI decode batches (config-2 model)")
     ap.add_argument("--seq-order", choices=["drawn", "snake"], default="drawn",
                     help="decode workloads, diagnostic: keep the drawn order of context lengths, or hand the batch over "
                          "sorted so that slots 256 / Hkv apart (the two workgroups of a CU) hold a long and a short one")
@@ -1139,6 +1141,144 @@ def bench_prefill_shapes(args):
                          "frac": round(best["TFLOPs"] / 2500.0, 4), "traffic": None}}
 
 
+def bench_timeline(args):
+    """Where a launch's time goes, per workgroup: the attention kernels stamp the GPU's 100 MHz counter at
+    fixed points of every workgroup's life (mkv_diag_timeline); this workload runs ONE stamped launch per
+    shape -- prefill batches (--prefill-shapes, whole prompts only) and decode batches (--timeline-decode,
+    BATCHxLO-HI on the config-2 model, fused append, rows in the balanced order) -- and reports, in
+    microseconds from the first workgroup's entry, the distribution of each point, of the phases between
+    them, and of the moment each CU is done (workgroups w and w + 256 share a CU while a grid is one round of
+    two workgroups per CU)."""
+    import ctypes as C
+    import torch
+    from morphserve_amd import _capi
+    from morphserve_amd.worker.kernels.paged_attn import choose_split
+
+    dev = torch.device("cuda:0")
+    lib = _capi.lib()
+    P = 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+
+    def q3(x):
+        x = x.double()
+        return {"min": round(float(x.min()), 2), "p10": round(float(x.quantile(0.1)), 2),
+                "median": round(float(x.median()), 2), "p90": round(float(x.quantile(0.9)), 2),
+                "max": round(float(x.max()), 2)}
+
+    def stamped(run, nwg, names, phases):
+        for _ in range(5):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        buf = torch.zeros(nwg * P, dtype=torch.int64, device=dev)
+        _capi.check(lib.mkv_diag_timeline(buf.data_ptr(), nwg))
+        try:
+            run()
+            torch.cuda.synchronize()
+        finally:
+            _capi.check(lib.mkv_diag_timeline(None, 0))
+        d = buf.cpu().view(nwg, P).double()
+        d = d[d[:, 0] > 0]
+        t0 = d[:, 0].min()
+        row = {"us_per_launch_unstamped": round(e0.elapsed_time(e1) / 20 * 1e3, 2), "workgroups": int(d.shape[0])}
+        row["points_us"] = {nm: q3((d[d[:, k] > 0, k] - t0) / 100.0) for k, nm in enumerate(names) if (d[:, k] > 0).any()}
+        row["phases_us"] = {}
+        for a, b, nm in phases:
+            m = (d[:, a] > 0) & (d[:, b] > 0)
+            if m.any():
+                row["phases_us"][nm] = q3((d[m, b] - d[m, a]) / 100.0)
+        last = d.max(dim=1).values
+        fin = (last - t0) / 100.0
+        row["workgroup_done_us"] = {"mean": round(float(fin.mean()), 2), "max": round(float(fin.max()), 2)}
+        if d.shape[0] == 512:
+            cu = torch.maximum(fin[:256], fin[256:])
+            row["cu_done_us"] = {**q3(cu), "mean": round(float(cu.mean()), 2)}
+            row["cu_done_mean_us_by_xcd"] = [round(float(cu[x::8].mean()), 2) for x in range(8)]
+        return row
+
+    rows = {}
+    H, D = 32, 128
+    for shape in [x for x in args.prefill_shapes.split(",") if x and "+" not in x]:
+        nseq, ln = (int(x) for x in shape.split("x"))
+        T = nseq * ln
+        q, k, v = (torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g) for _ in range(3))
+        o = torch.empty_like(q)
+        starts = torch.arange(nseq, dtype=torch.int32, device=dev) * ln
+        lens = torch.full((nseq,), ln, dtype=torch.int32, device=dev)
+
+        def run():
+            _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), starts.data_ptr(),
+                                             lens.data_ptr(), nseq, ln, H, H, D, D ** -0.5, _capi.current_stream()))
+        names = ["entry", "first tile staged", "tiles done", "written", "second part: first tile staged",
+                 "second part: tiles done", "second part: written"]
+        phases = [(0, 1, "entry -> first tile staged"), (1, 2, "first part: key tiles"), (2, 3, "first part: output"),
+                  (2, 4, "first part done -> second part staged"), (4, 5, "second part: key tiles"),
+                  (5, 6, "second part: output")]
+        rows["prefill " + shape] = stamped(run, 1 << 16, names, phases)
+        del q, k, v, o
+
+    L, HQ, HKV, B = 32, 32, 8, 16
+    nb = args.pool_blocks or 16384
+    kc = torch.randn((nb, L, HKV, B, D), dtype=torch.float16, device=dev, generator=g)
+    vc = torch.randn((nb, L, HKV, B, D), dtype=torch.float16, device=dev, generator=g)
+    pool = _capi.make_pool(kc, vc)
+    rng = np.random.default_rng(args.seed)
+    for shape in [x for x in args.timeline_decode.split(",") if x]:
+        n_s, ctx = shape.split("x")
+        N = int(n_s)
+        lo, hi = (int(x) for x in ctx.split("-")) if "-" in ctx else (int(ctx), int(ctx))
+        lens = rng.integers(lo, hi + 1, size=N).astype(np.int32)
+        nblk = (lens + B - 1) // B
+        mbs = int(nblk.max()) + 1
+        assert int(nblk.sum()) <= nb, "pool too small for this batch"
+        perm = rng.permutation(nb)
+        table = np.zeros((N, mbs), dtype=np.int32)
+        pos = 0
+        for i in range(N):
+            table[i, :nblk[i]] = perm[pos:pos + nblk[i]]
+            pos += nblk[i]
+        bt = torch.from_numpy(table).to(dev)
+        lens_t = torch.from_numpy(lens).to(dev)
+        ids = torch.arange(N, dtype=torch.int32, device=dev)
+        q = torch.randn((N, HQ, D), dtype=torch.float16, device=dev, generator=g)
+        kn = torch.randn((N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+        vn = torch.randn((N, HKV, D), dtype=torch.float16, device=dev, generator=g)
+        tps, splits = choose_split(N, HKV, int(lens.max()), B)
+        mid_o = torch.empty(N * HQ * splits * D, dtype=torch.float32, device=dev)
+        mid_lse = torch.empty(N * HQ * splits, dtype=torch.float32, device=dev)
+        order = torch.empty(N, dtype=torch.int32, device=dev)
+        o = torch.empty((N, HQ * D), dtype=torch.float16, device=dev)
+        if N >= 2:
+            _capi.check(lib.mkv_decode_order(lens_t.data_ptr(), N, HKV, order.data_ptr(), _capi.current_stream()))
+
+        def run():
+            _capi.check(lib.mkv_decode_attn_ordered(
+                q.data_ptr(), o.data_ptr(), C.byref(pool), bt.data_ptr(), mbs, ids.data_ptr(), lens_t.data_ptr(),
+                order.data_ptr() if N >= 2 else None, N, HQ, D ** -0.5, 5, tps, splits, mid_o.data_ptr(),
+                mid_lse.data_ptr(), kn.data_ptr(), vn.data_ptr(), None, None, _capi.current_stream()))
+        names = ["entry", "before the block loop", "blocks done", "stored"]
+        phases = [(0, 1, "entry -> block loop"), (1, 2, "block loop"), (2, 3, "merge of the waves and store")]
+        row = stamped(run, splits * HKV * N, names, phases)
+        row["splits"] = splits
+        row["note"] = "us_per_launch_unstamped includes the merge launch when splits > 1"
+        row["algorithmic_MB"] = round(sum(decode_bytes_per_layer(lens, N, HQ, HKV, D, B)) / 1e6, 1)
+        rows["decode " + shape] = row
+    first = next(iter(rows.values()))
+    return {"metric": "per-workgroup timeline of the attention kernels, 1 MI355X", "value": first["us_per_launch_unstamped"],
+            "unit": "us/launch", "n_gpus": 1, "steps": 1, "warmup": 5, "ms_per_step": first["us_per_launch_unstamped"] / 1e3,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
+            "data": "synthetic",
+            "config": {"workload": f"timeline: prefill {args.prefill_shapes} (MHA 32/32), decode {args.timeline_decode} "
+                                   f"(config-2 model, pool {nb} blocks); one stamped launch each"},
+            "shapes": rows}
+
+
 def bench_placement_probe(args):
     """Does the rate follow the ALLOCATION?  Four KV pools of 32 GiB in one process, the same config-2 decode
     batch (same tables, same q / k / v) run on each in turn, twice; then a sequential 1 GiB copy inside each
@@ -1371,7 +1511,8 @@ def main():
              "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
              "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
-             "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving}
+             "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving,
+             "timeline": bench_timeline}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
         # the second target of the path in the same process and the same JSON line: the decode pool is gone

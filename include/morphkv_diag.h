@@ -50,6 +50,19 @@ int mkv_set_prefill_variant(int32_t waves);
 int mkv_diag_mfma_loop(int32_t mode, int32_t iters, const void* data, void* sink, double* flops,
                        void* stream);
 
+/* Per-workgroup time stamps of the attention kernels.  buf: device memory of
+ * max_workgroups * MKV_TIMELINE_POINTS int64, zeroed by the caller; NULL switches
+ * the stamps off.  While set, every launch of the prefill kernel and of the decode
+ * phase-1 kernels whose grid has at most max_workgroups workgroups makes thread 0
+ * of workgroup w (linear id, x fastest) store the GPU's constant-rate 100 MHz
+ * counter into buf[w * MKV_TIMELINE_POINTS + k] at point k of its life -- prefill:
+ * 0 entry, 1 first key tile staged, 2 key tiles done, 3 output written, 4-6 the
+ * same three for the workgroup's second query tile; decode: 0 entry, 1 before the
+ * block loop, 2 blocks done, 3 output stored.  Later launches overwrite earlier
+ * ones: set it around ONE launch and synchronise. */
+#define MKV_TIMELINE_POINTS 8
+int mkv_diag_timeline(void* buf, int64_t max_workgroups);
+
 /* When enabled, every launch of the kernels above is bracketed by a
  * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
  * returns the launch count and summed duration since the last reset. */

@@ -76,4 +76,19 @@ __host__ __device__ __forceinline__ int64_t pool_total_blocks(const mkv_pool& p)
 
 static inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
+// ---- per-workgroup time stamps (diagnostic, mkv_diag_timeline) -----------------
+// The attention launchers hand their kernels the buffer set by mkv_diag_timeline when it holds the
+// launch's workgroups, NULL otherwise.  With a buffer, thread 0 of workgroup w stores the constant-rate
+// 100 MHz counter at point k of its life into buf[w * MKV_TIMELINE_POINTS + k]; without one a mark is
+// a scalar test and a branch.
+long long* timeline_buffer(int64_t workgroups);
+
+__device__ __forceinline__ void timeline_mark(long long* tl, int64_t wg, int k) {
+    if (tl != nullptr && threadIdx.x == 0) {
+        unsigned long long t;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t));
+        tl[wg * MKV_TIMELINE_POINTS + k] = (long long)t;
+    }
+}
+
 }  // namespace mkv

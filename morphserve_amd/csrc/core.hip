@@ -48,6 +48,14 @@ int check_pool(const mkv_pool* p) {
     return MKV_OK;
 }
 
+// ---- per-workgroup time stamps -----------------------------------------------------
+static long long* g_timeline = nullptr;
+static int64_t g_timeline_wgs = 0;
+
+long long* timeline_buffer(int64_t workgroups) {
+    return (g_timeline != nullptr && workgroups <= g_timeline_wgs) ? g_timeline : nullptr;
+}
+
 // ---- profiling ---------------------------------------------------------------
 struct ProfRec {
     hipEvent_t start, stop;
@@ -100,6 +108,14 @@ int mkv_pool_set_strided(mkv_pool* pool, void* k_new0, void* v_new0,
         pool->v_seg[j] = (char*)v_new0 - back;
     }
     for (int j = num_segments; j < MKV_MAX_SEGMENTS; ++j) pool->k_seg[j] = pool->v_seg[j] = nullptr;
+    return MKV_OK;
+}
+
+int mkv_diag_timeline(void* buf, int64_t max_workgroups) {
+    MKV_REQUIRE(buf == nullptr || max_workgroups > 0, "max_workgroups must be positive with a buffer");
+    MKV_REQUIRE(((uintptr_t)buf & 7) == 0, "the time stamp buffer must be 8-byte aligned");
+    mkv::g_timeline = (long long*)buf;
+    mkv::g_timeline_wgs = buf ? max_workgroups : 0;
     return MKV_OK;
 }
 

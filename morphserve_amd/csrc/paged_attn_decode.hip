@@ -182,7 +182,10 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ v_new,
     const uint4* __restrict__ cos_t,    // [n, D/2] fp16 or NULL: rotate q and the new k row on the way in
     const uint4* __restrict__ sin_t,
-    const int32_t* __restrict__ order) {   // [n] or NULL: batch row taken by each slot of the grid
+    const int32_t* __restrict__ order,     // [n] or NULL: batch row taken by each slot of the grid
+    long long* __restrict__ timeline) {    // per-workgroup time stamps (diagnostic) or NULL
+    const int64_t wg_id = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    timeline_mark(timeline, wg_id, 0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -195,7 +198,12 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const int len = seq_lens[i];
     const int nblk = (int)min((int64_t)((len + kB - 1) / kB), max_blocks_per_seq);   // never read past the table row
     const int blk_begin = split * blocks_per_split;
-    if (blk_begin >= nblk) return;                      // uniform over the workgroup
+    if (blk_begin >= nblk) {
+        // nothing of the sequence lies in this split: the merge must see an empty slot, not stale scratch
+        if (gridDim.x > 1 && threadIdx.x < G)
+            mid_lse[((int64_t)i * Hq + kvh * G + threadIdx.x) * max_splits + split] = kNegBig;
+        return;                                         // uniform over the workgroup
+    }
     // the last launched split also takes whatever lies beyond it, so an
     // under-estimated max_splits costs balance, never tokens
     const int blk_end = (split == (int)gridDim.x - 1) ? nblk : min(blk_begin + blocks_per_split, nblk);
@@ -239,6 +247,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     // is handled apart, so the main loop carries no masking and no branches around
     // its loads: the loads of block t+1 are issued before block t is consumed and
     // stay in flight behind it.
+    timeline_mark(timeline, wg_id, 1);
     const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
     const int n_it = max(0, (blk_end - my_first + 3) >> 2);
     // blocks [0, nblk_full) hold 16 valid tokens and need no special care; with a
@@ -352,6 +361,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     }
 
     // ---- merge the four waves through LDS ------------------------------------------
+    timeline_mark(timeline, wg_id, 2);
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
     __shared__ float sm_l[4][G];
@@ -369,6 +379,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     __syncthreads();
     merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
                              max_splits);
+    timeline_mark(timeline, wg_id, 3);
 }
 
 // ---- matrix-core variant for GQA groups (G >= 4) -----------------------------------
@@ -406,7 +417,10 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     int64_t max_blocks_per_seq, const int32_t* __restrict__ seq_ids,
     const int32_t* __restrict__ seq_lens, float scale2, int32_t layer, int32_t blocks_per_split,
     int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new,
-    const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t, const int32_t* __restrict__ order) {
+    const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t, const int32_t* __restrict__ order,
+    long long* __restrict__ timeline) {
+    const int64_t wg_id = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    timeline_mark(timeline, wg_id, 0);
     __shared__ __attribute__((aligned(16))) char stage[4][2][kLdsTile];
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
@@ -425,7 +439,12 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     const int len = seq_lens[i];
     const int nblk = (int)min((int64_t)((len + kB - 1) / kB), max_blocks_per_seq);
     const int blk_begin = split * blocks_per_split;
-    if (blk_begin >= nblk) return;
+    if (blk_begin >= nblk) {
+        // nothing of the sequence lies in this split: the merge must see an empty slot, not stale scratch
+        if (gridDim.x > 1 && threadIdx.x < G)
+            mid_lse[((int64_t)i * Hq + kvh * G + threadIdx.x) * max_splits + split] = kNegBig;
+        return;                                         // uniform over the workgroup
+    }
     const int blk_end = (split == (int)gridDim.x - 1) ? nblk : min(blk_begin + blocks_per_split, nblk);
     const int64_t seq = seq_ids[i];
     const int32_t* row = block_table + seq * max_blocks_per_seq;
@@ -559,6 +578,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         wave_lds_fence();                            // reads done before the next tile is staged
     };
 
+    timeline_mark(timeline, wg_id, 1);
     const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
     const int n_it = max(0, (blk_end - my_first + 3) >> 2);
     // blocks [0, nblk_full) hold 16 valid tokens; the final block takes the careful
@@ -603,6 +623,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         }
     }
 
+    timeline_mark(timeline, wg_id, 2);
     float l_tot = l_run + __shfl_xor(l_run, 16);
     l_tot += __shfl_xor(l_tot, 32);
     if (n < G) {
@@ -618,64 +639,78 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     __syncthreads();
     merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
                              max_splits);
+    timeline_mark(timeline, wg_id, 3);
 }
 
-// Phase 2: one workgroup of 128 threads per (sequence, q head): log-sum-exp merge
-// of the per-split partials, cast to fp16.
+// Phase 2: log-sum-exp merge of the per-split partials, cast to fp16.  Both kernels read
+// ALL max_splits slots of their (sequence, q head) -- phase 1 marks the slots of splits beyond a
+// sequence's end with kNegBig -- so nothing here waits for the sequence's length: the partials and
+// their log-sum-exps are requested together, one trip to memory between launch and store.
+__device__ __forceinline__ bool slot_live(float lse) { return lse > 0.5f * kNegBig; }
+
+// Up to 8 splits: one workgroup of 128 threads per (sequence, q head), thread = output dim.
 __global__ __launch_bounds__(128) void attn_decode_phase2(
     const float* __restrict__ mid_o, const float* __restrict__ mid_lse, __half* __restrict__ o,
-    const int32_t* __restrict__ seq_lens, int32_t num_q_heads, int32_t tokens_per_split,
-    int32_t max_splits) {
+    int32_t num_q_heads, int32_t max_splits) {
     const int i = blockIdx.y;
     const int hq = blockIdx.x;
     const int d = threadIdx.x;
-    const int len = seq_lens[i];
-    const int ns = min((len + tokens_per_split - 1) / tokens_per_split, max_splits);
     const int64_t base = ((int64_t)i * num_q_heads + hq) * max_splits;
-    float m = kNegBig, l = 0.f, acc = 0.f;
-    for (int s = 0; s < ns; ++s) {
-        const float lse = mid_lse[base + s];
-        const float v = mid_o[(base + s) * kD + d];
-        const float m_new = fmaxf(m, lse);
-        const float old = fast_exp2(m - m_new);
-        const float e = fast_exp2(lse - m_new);
-        acc = acc * old + e * v;
-        l = l * old + e;
-        m = m_new;
+    float lse[8], v[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int sc = min(s, max_splits - 1);                  // slots past the last re-read it (and are ignored)
+        lse[s] = mid_lse[base + sc];
+        v[s] = mid_o[(base + sc) * kD + d];
     }
-    o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(ns > 0 ? acc / l : 0.f);
+    float m = kNegBig;
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        if (s < max_splits) m = fmaxf(m, lse[s]);
+    float l = 0.f, acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        if (s < max_splits && slot_live(lse[s])) {              // an empty slot's partial is never touched
+            const float e = fast_exp2(lse[s] - m);
+            l += e;
+            acc = fmaf(e, v[s], acc);
+        }
+    }
+    o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(l > 0.f ? acc / l : 0.f);
 }
 
-// Phase 2 for many splits (long contexts at small batch): the serial loop above is one
-// dependent chain of loads per thread.  Here a workgroup of four waves takes one
-// (sequence, q head); splits are consumed 64 at a time: every wave reads the chunk's 64
-// log-sum-exps (one per lane), reduces them to the chunk max and the weights
-// w_s = exp2(lse_s - max) -- the same values in all four waves --, then wave w gathers the
-// partials of splits w, w+4, ... with SIXTEEN independent 8-byte loads per lane in flight
-// (lane l owns dims 2l, 2l+1; out-of-range slots re-read the chunk's last split with weight
-// zero).  The four waves' sums meet in LDS.
+// More than 8 splits (long contexts at small batch): a workgroup of four waves takes one
+// (sequence, q head); slots are consumed 64 at a time.  Wave w requests the partials of slots
+// w, w+4, ... with SIXTEEN independent 8-byte loads per lane (lane l owns dims 2l, 2l+1) and, behind
+// them, the chunk's 64 log-sum-exps (one per lane); the loads return while the chunk max and the
+// weights w_s = exp2(lse_s - max) -- the same values in all four waves -- are formed with wave
+// reductions.  The four waves' sums meet in LDS.
 __global__ __launch_bounds__(256) void attn_decode_phase2_wide(
     const float* __restrict__ mid_o, const float* __restrict__ mid_lse, __half* __restrict__ o,
-    const int32_t* __restrict__ seq_lens, int32_t num_q_heads, int32_t tokens_per_split,
-    int32_t max_splits) {
+    int32_t num_q_heads, int32_t max_splits) {
     __shared__ float part[4][kD];
     const int i = blockIdx.y;
     const int hq = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int len = seq_lens[i];
-    const int ns = min((len + tokens_per_split - 1) / tokens_per_split, max_splits);
     const int64_t base = ((int64_t)i * num_q_heads + hq) * max_splits;
     float m = kNegBig, l = 0.f, a0 = 0.f, a1 = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += 64) {
-        const int cnt = min(64, ns - s0);
-        const float lse = lane < cnt ? mid_lse[base + s0 + lane] : kNegBig;
-        float mc = lse;
+    for (int s0 = 0; s0 < max_splits; s0 += 64) {
+        const int cnt = min(64, max_splits - s0);
+        float2 v[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int jc = min(wave + 4 * e, cnt - 1);                 // wave-uniform
+            v[e] = *(const float2*)(mid_o + (base + s0 + jc) * kD + 2 * lane);
+        }
+        const float lse = mid_lse[base + s0 + min(lane, cnt - 1)];
+        const bool live = lane < cnt && slot_live(lse);
+        float mc = live ? lse : kNegBig;
 #pragma unroll
         for (int sh = 32; sh >= 1; sh >>= 1) mc = fmaxf(mc, __shfl_xor(mc, sh));
         const float m_new = fmaxf(m, mc);
         const float old = fast_exp2(m - m_new);
-        const float wgt = lane < cnt ? fast_exp2(lse - m_new) : 0.f;
+        const float wgt = live ? fast_exp2(lse - m_new) : 0.f;
         float wsum = wgt;
 #pragma unroll
         for (int sh = 32; sh >= 1; sh >>= 1) wsum += __shfl_xor(wsum, sh);
@@ -683,19 +718,14 @@ __global__ __launch_bounds__(256) void attn_decode_phase2_wide(
         a0 *= old;
         a1 *= old;
         m = m_new;
-        float2 v[16];
-        float w[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int j = wave + 4 * e;                                // wave-uniform
-            const int jc = min(j, cnt - 1);
-            w[e] = j < cnt ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wgt), jc)) : 0.f;
-            v[e] = *(const float2*)(mid_o + (base + s0 + jc) * kD + 2 * lane);
-        }
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            a0 = fmaf(w[e], v[e].x, a0);
-            a1 = fmaf(w[e], v[e].y, a1);
+            const float w = j < cnt ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wgt), min(j, cnt - 1))) : 0.f;
+            if (w != 0.f) {                                            // wave-uniform: an empty slot's partial is never touched
+                a0 = fmaf(w, v[e].x, a0);
+                a1 = fmaf(w, v[e].y, a1);
+            }
         }
     }
     part[wave][2 * lane] = a0;
@@ -704,7 +734,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase2_wide(
     if (threadIdx.x < kD) {
         const int d = threadIdx.x;
         const float acc = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
-        o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(ns > 0 ? acc / l : 0.f);
+        o[((int64_t)i * num_q_heads + hq) * kD + d] = __float2half(l > 0.f ? acc / l : 0.f);
     }
 }
 
@@ -722,18 +752,19 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
     // size (up to the 16 columns of a matrix tile) runs on the matrix cores
     constexpr bool has_valu = G == 1 || G == 2 || G == 4 || G == 8;
     const bool mfma = !has_valu || g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
+    long long* timeline = timeline_buffer((int64_t)grid.x * grid.y * grid.z);
     if (mfma) {
         hipLaunchKernelGGL(attn_decode_phase1_mfma<G>, grid, dim3(256), 0, s, (const uint4*)q,
                            (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
                            max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
                            max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
-                           (const uint4*)sin_t, order);
+                           (const uint4*)sin_t, order, timeline);
     } else if constexpr (has_valu) {
         hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
                            (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
                            seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
                            (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t,
-                           order);
+                           order, timeline);
     }
 }
 
@@ -822,11 +853,11 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
         if (max_splits > 8) {       // a long chain of partials per head: the gather-in-parallel merge
             hipLaunchKernelGGL(mkv::attn_decode_phase2_wide, dim3((unsigned)num_q_heads, (unsigned)n),
                                dim3(256), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
-                               seq_lens, num_q_heads, tokens_per_split, max_splits);
+                               num_q_heads, max_splits);
         } else {
             hipLaunchKernelGGL(mkv::attn_decode_phase2, dim3((unsigned)num_q_heads, (unsigned)n),
                                dim3(128), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
-                               seq_lens, num_q_heads, tokens_per_split, max_splits);
+                               num_q_heads, max_splits);
         }
         MKV_HIP(hipGetLastError());
     }

@@ -71,6 +71,7 @@ struct PrefillArgs {
     int32_t num_seqs;
     int32_t num_q_tiles;          // ceil(max_len / query rows per workgroup)
     int32_t pair_tiles;           // 1: a workgroup takes two query tiles (i-th from the end, i-th from the start); 0: one
+    long long* timeline;          // per-workgroup time stamps (diagnostic) or NULL
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -91,7 +92,8 @@ __device__ __forceinline__ float max_over_groups(float x) {
     auto b = __builtin_amdgcn_permlane32_swap(yi, yi, false, false);
     return fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
 }
-template <bool PAGED, int WAVES>
+// TL: the instance that takes per-workgroup time stamps (launched only while mkv_diag_timeline holds a buffer)
+template <bool PAGED, int WAVES, bool TL>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
     constexpr int kThreads = 64 * WAVES;
     constexpr int kQTile = 16 * kU * WAVES;                    // query rows per workgroup
@@ -102,6 +104,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     __shared__ __attribute__((aligned(16))) char v_lds[2 * kVBuf];
 
     const int tid = threadIdx.x;
+    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 0);
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int m = lane & 15;          // query row of a column tile (B / C), key or dim row (A)
@@ -454,6 +457,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         __syncthreads();
     }
     carried = false;
+    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 1 + 3 * part);
     for (int it = 0; it + 1 < num_tiles; it += 2) {
         iteration(it, Set0{}, Set1{});
         if (it + 2 < num_tiles) iteration(it + 1, Set1{}, Set0{});
@@ -481,6 +485,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         }
         __syncthreads();                              // every read of the staged tiles is done
     }
+    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 2 + 3 * part);
 
     // Output: a lane holds four dims of sixteen rows' worth of 8-byte pieces; the column tile goes
     // through this wave's corner of the idle V buffer (rows 288 bytes apart: conflict-free 8-byte
@@ -509,6 +514,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         if (more) stage_tile(0, Set0{});
         if (follows) __syncthreads();                 // the next part's staging may reuse every buffer
         if (more) carried = true;
+        if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 3 + 3 * part);
     }
   }   // part
 }
@@ -542,18 +548,23 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
     args.pair_tiles = (g_prefill_pairing == 1 || (g_prefill_pairing == 0 && !unpair)) ? 1 : 0;
     const int64_t unpaired = ((pairs8 / 8 * args.num_q_tiles + 31) / 32 * 32) * 8;      // whole runs of 32 slots per XCD
     dim3 grid((unsigned)(args.pair_tiles ? paired : unpaired));
+    args.timeline = timeline_buffer(grid.x);
     static const mkv_pool empty = {};
     {
         ProfScope prof(MKV_K_PREFILL_ATTN, s);
+        const bool tl = args.timeline != nullptr;
+#define MKV_LAUNCH(P, W, T, TH, PL) \
+    hipLaunchKernelGGL((prefill_attn_kernel<P, W, T>), grid, dim3(TH), 0, s, args, PL)
         if (paged && waves == 8) {
-            hipLaunchKernelGGL((prefill_attn_kernel<true, 8>), grid, dim3(512), 0, s, args, *pool);
+            if (tl) MKV_LAUNCH(true, 8, true, 512, *pool); else MKV_LAUNCH(true, 8, false, 512, *pool);
         } else if (paged) {
-            hipLaunchKernelGGL((prefill_attn_kernel<true, 4>), grid, dim3(256), 0, s, args, *pool);
+            if (tl) MKV_LAUNCH(true, 4, true, 256, *pool); else MKV_LAUNCH(true, 4, false, 256, *pool);
         } else if (waves == 8) {
-            hipLaunchKernelGGL((prefill_attn_kernel<false, 8>), grid, dim3(512), 0, s, args, empty);
+            if (tl) MKV_LAUNCH(false, 8, true, 512, empty); else MKV_LAUNCH(false, 8, false, 512, empty);
         } else {
-            hipLaunchKernelGGL((prefill_attn_kernel<false, 4>), grid, dim3(256), 0, s, args, empty);
+            if (tl) MKV_LAUNCH(false, 4, true, 256, empty); else MKV_LAUNCH(false, 4, false, 256, empty);
         }
+#undef MKV_LAUNCH
     }
     MKV_HIP(hipGetLastError());
     return MKV_OK;
