@@ -23,7 +23,8 @@ int mkv_set_decode_variant(int32_t variant);
 
 /* Experiments and tests: pin the prefill kernel's workgroup shape.  Bits 0-7:
  * 0 = by the call (eight waves / 256 query rows per workgroup from 2048-token
- * chunks whose grid still covers the chip, four waves / 128 rows otherwise),
+ * chunks, or from 256-row chunks over at least 512 cached tokens, where that grid
+ * still covers the chip; four waves / 128 rows otherwise),
  * 4 or 8 = always that shape.  Bits 8-9: 0 = a workgroup takes two query tiles
  * of its sequence unless the grid would be too small, 1 = always two, 2 = always
  * one. */

@@ -535,7 +535,9 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
     // shorter chunk on (8 x 512 over 2048 cached tokens: 217 -> 207 us, 4 x 1024 over 4096: 388 -> 349 us)
     const bool many_keys = max_len >= kLongPrompt ||
                            (max_len >= kChunkRows && max_prefix >= kLongPrefix && max_len + max_prefix >= 1024);
-    const bool long_and_wide = many_keys && pairs8 * ((cdiv(max_len, 16 * kU * 8) + 1) / 2) >= 256;
+    // (over the batch's own k, v a grid of exactly one eight-wave workgroup per CU loses to two four-wave ones:
+    // 2 x 2048 tokens 86 against 79 us, 1 x 4096 158 against 142 us; from one and a half per CU on it wins)
+    const bool long_and_wide = many_keys && pairs8 * ((cdiv(max_len, 16 * kU * 8) + 1) / 2) >= (paged ? 256 : 320);
     const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (long_and_wide ? 8 : 4);
     const int q_tile = 16 * kU * waves;
     args.num_q_tiles = cdiv(max_len, q_tile);
