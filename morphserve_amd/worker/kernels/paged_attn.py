@@ -59,12 +59,13 @@ def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
     return cur
 
 
-def _decode_order(infer_state, lens: torch.Tensor, n: int, num_kv_heads: int) -> Optional[torch.Tensor]:
+def _decode_order(infer_state, lens: torch.Tensor, n: int, num_kv_heads: int, splits: int) -> Optional[torch.Tensor]:
     """The balanced order of this batch's rows, computed by one small launch the first time a layer asks
     for it and kept on ``infer_state`` for the other layers of the step (it depends on the lengths only).
     An order that has gone stale -- lengths updated in place -- is still a permutation, so the outputs
-    do not depend on it; only the balance does."""
-    if not BALANCED_ORDER or n < 2 or n > 4096:
+    do not depend on it; only the balance does.  A batch that is cut into splits needs none: its workgroups
+    carry equal token counts already."""
+    if not BALANCED_ORDER or n < 2 or n > 4096 or splits > 1:
         return None
     key = (lens.data_ptr(), n, num_kv_heads)
     cached = getattr(infer_state, "_morphkv_decode_order", None)
@@ -132,7 +133,7 @@ def decode_append_and_attend(
     mid_o, mid_lse = (None, None)
     if splits > 1:
         mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
-    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads, splits)
     _capi.check(_capi.lib().mkv_decode_attn_ordered(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
         infer_state.seq_ids.data_ptr(), infer_state.decoding_seq_lens.data_ptr(), _capi.ptr(order), n, hq,
@@ -176,7 +177,7 @@ def decode_rope_append_and_attend(
     mid_o, mid_lse = (None, None)
     if splits > 1:
         mid_o, mid_lse = _get_scratch(q.device, n, hq, splits, d)
-    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads, splits)
     _capi.check(_capi.lib().mkv_decode_attn_ordered(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1],
         infer_state.seq_ids.data_ptr(), infer_state.decoding_seq_lens.data_ptr(), _capi.ptr(order), n, hq,
@@ -223,7 +224,7 @@ def paged_attention(
     seq_ids_ptr = infer_state.seq_ids.data_ptr() + ids_off
     lens_ptr = infer_state.decoding_seq_lens.data_ptr()
     pending = _deferred.take(k_cache, v_cache, block_table, seq_ids_ptr, lens_ptr, n, cur_layer)
-    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads)
+    order = _decode_order(infer_state, infer_state.decoding_seq_lens, n, model_config.num_kv_heads, splits)
     # a pending append: the decode rows store_kvcache was given for this layer are appended by this launch
     _capi.check(lib.mkv_decode_attn_ordered(
         q.data_ptr(), o.data_ptr(), C.byref(pool), block_table.data_ptr(), block_table.shape[1], seq_ids_ptr,
