@@ -151,9 +151,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 
   // State that outlives a part: while the last key tile of part 0 is consumed, q and the first K/V
   // tile(s) of part 1 are already requested, so the second part starts without a trip to memory.
-  constexpr int kFetchStepsO = (kKTile * 16) / (64 * WAVES);
   v8h qb[kU][4];
-  v4u kreg[WAVES == 8 ? 2 : 1][kFetchStepsO], vreg[WAVES == 8 ? 2 : 1][kFetchStepsO];
+  v4u kreg[kSets][kFetchSteps], vreg[kSets][kFetchSteps];     // staging registers: one set per tile in flight
   int32_t tile_ids = 0;
   int f_kv_len = 0;                   // the fetch side's view: keys of the part whose tiles are being requested
   uint32_t last_off = 0, next_off = 0;
@@ -223,7 +222,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     // probabilities are zero); unmapped table entries read as zeros.
     // Contiguous source: one uniform base per (sequence, kv head) plus a 32-bit byte offset
     // per lane that advances by a constant per tile (the launcher bounds len * Hkv * 256).
-    static_assert(kFetchSteps == kFetchStepsO, "staging register count");
     const uint32_t row_stride = (uint32_t)Hkv * (kPD * 2);
     const char* k_src = PAGED ? nullptr : (const char*)a.k + (start * Hkv + kvh) * (int64_t)(kPD * 2);
     const char* v_src = PAGED ? nullptr : (const char*)a.v + (start * Hkv + kvh) * (int64_t)(kPD * 2);
@@ -467,9 +465,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         const int key0 = it * kKTile;
         const bool active = wave_has_rows && key0 <= wave_max_pos;
         uint4 kf_first[4];
-        if (active) first_frags(it & 1, kf_first);
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) {                                   // both staging sets are idle: the next part's first tile(s)
+        auto request_next_part = [&]() {              // both staging sets are idle: the next part's first tile(s)
             int kvl = nx_kv_len;
             asm volatile("" : "+s"(kvl));             // keeps the next part's addresses out of the tile loop's registers
             const int nx_tiles = (kvl + kKTile - 1) / kKTile;
@@ -477,11 +473,24 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             nx_kv_len = 0;
             fetch_tile(0, Set0{});
             if (kSets == 2 && nx_tiles > 1) fetch_tile(kKTile, Set1{});
-        }
-        if (active) {
-            tile_body(std::true_type{}, it & 1, key0, kf_first, more ? nx_q0 : -1);
-        } else if (more) {
-            load_q(nx_q0);
+        };
+        // Contiguous source: the request's address arithmetic covers the latency of the first K fragments, and
+        // the next part's q is asked for inside the tile, once the scores have released its registers.  The
+        // paged source's arithmetic needs those registers itself (fragments held across it would spill, and
+        // their reload would wait for the very loads just issued): request first, q after the tile.
+        if (PAGED) {
+            if (more) request_next_part();
+            if (active) {
+                first_frags(it & 1, kf_first);
+                tile_body(std::true_type{}, it & 1, key0, kf_first, -1);
+            }
+            if (more) load_q(nx_q0);
+        } else {
+            if (active) first_frags(it & 1, kf_first);
+            __builtin_amdgcn_sched_barrier(0);
+            if (more) request_next_part();
+            if (active) tile_body(std::true_type{}, it & 1, key0, kf_first, more ? nx_q0 : -1);
+            else if (more) load_q(nx_q0);
         }
         __syncthreads();                              // every read of the staged tiles is done
     }
