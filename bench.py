@@ -881,7 +881,7 @@ def bench_mixed(args):
                            f"{chunk_flops / (chunk_ms * 1e-3) / 1e12:.1f} TFLOP/s",
         "rotary_then_store_ms": round(rope_two_ms, 5), "rotary_store_fused_ms": round(rope_fused_ms, 5),
         "rotary_store_fused_GBs": round(rope_bytes / (rope_fused_ms * 1e-3) / 1e9, 1),
-        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false, 4>", "achieved": round(tflops, 1),
+        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false, 4, false>", "achieved": round(tflops, 1),
                      "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4),
                      "timing": "one event pair around 50 back-to-back launches of this kernel only",
                      "traffic": measured_traffic(f"cfg4_mixed prefill=8x512 seed={args.seed}")},
