@@ -102,7 +102,18 @@ def test_random_prefill_and_chunked_prefill(cuda, seed):
     rng = np.random.default_rng(3000 + seed)
     Hq, Hkv = HEADS[int(rng.integers(len(HEADS)))]
     n = int(rng.integers(1, 6))
-    lens = _lens(rng, n, int(rng.choice([40, 200, 700])))
+    lens = _lens(rng, n, int(rng.choice([40, 200, 700, 1300])))
+    # workgroup shape and tile pairing: the library's choice, or pinned (small grids never pick the paired and the
+    # 256-row shapes by themselves): bits 0-7 waves, bits 8-9 pairing forced on (1) / off (2)
+    variant = int(rng.choice([0, 4 | (1 << 8), 4 | (2 << 8), 8 | (1 << 8), 8 | (2 << 8)]))
+    _capi.check(_capi.lib().mkv_set_prefill_variant(variant))
+    try:
+        _random_prefill_case(cuda, seed, rng, Hq, Hkv, n, lens, variant)
+    finally:
+        _capi.check(_capi.lib().mkv_set_prefill_variant(0))
+
+
+def _random_prefill_case(cuda, seed, rng, Hq, Hkv, n, lens, variant):
     T = int(lens.sum())
     q = rand_f16(rng, T, Hq, 128)
     k = rand_f16(rng, T, Hkv, 128)
@@ -116,7 +127,7 @@ def test_random_prefill_and_chunked_prefill(cuda, seed):
                       o, model, engine, st)
     torch.cuda.synchronize()
     want = R.prefill_attention(q, k, v, starts, lens, 128 ** -0.5, math="np32")
-    assert_attn_close(o.cpu().numpy(), want, f"seed {seed}: prefill Hq={Hq} Hkv={Hkv} lens={lens.tolist()}")
+    assert_attn_close(o.cpu().numpy(), want, f"seed {seed}: prefill Hq={Hq} Hkv={Hkv} lens={lens.tolist()} variant={variant}")
 
     # the same prompts cut at a random point: the tail as a chunk over the cached head
     L = 2
