@@ -85,6 +85,8 @@ def parse_args():
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches; SEQSxTOKENS+PREFIX is a "
                          "batch of chunks over PREFIX tokens already in a paged cache")
+    ap.add_argument("--no-placement-tuning", action="store_true",
+                    help="decode workloads, diagnostic: the V pool starts at its allocation's base (no probing of offsets)")
     ap.add_argument("--prefill-kv-heads", type=int, default=32,
                     help="prefill_shapes workload, whole prompts: kv heads behind the 32 q heads (1 = every q head reads the "
                          "same K/V, which then always comes out of the L2s: the same matrix work without the K/V traffic)")
@@ -176,9 +178,11 @@ def bench_decode(args):
         vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq,
                              chunk_blocks=args.vmm_chunk_blocks)
         k_cache, v_cache = vmm_pool.k_cache, vmm_pool.v_cache
-    else:
-        k_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
-        v_cache = torch.zeros(shape, dtype=torch.float16, device=dev)
+        kv_placement = {"v_offset_bytes": 0, "tuned": False}
+    else:                                         # as ElasticKVPool creates them: two zeroed allocations, the V base
+        from morphserve_amd.kv_placement import allocate_kv_caches   # a few KiB in where the gather measures faster
+        k_cache, v_cache, kv_placement = allocate_kv_caches(num_blocks, shape[1:], dev, zero_init=True,
+                                                            tune=not args.no_placement_tuning)
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     live_t = torch.from_numpy(live).to(dev)
@@ -359,6 +363,7 @@ def bench_decode(args):
                                  else "the grid takes the rows as given")
                                 + (", lengths handed over pre-ordered (--seq-order snake)" if args.seq_order == "snake" else "")},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "kv_placement": kv_placement,
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
         "us_per_step": round(ms_per_step * 1e3, 2),
         **({"note": "latency-bound: one layer moves a few tens of MB, so a step is a few launch latencies long and "

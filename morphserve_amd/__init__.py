@@ -12,6 +12,7 @@ Drop-in names (reference file each mirrors):
 * ``model_config.LlamaModelConfig``                  MorphServe/model_config.py (attention geometry, ``get_kvslot_size``)
 * ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
 * ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
+* ``kv_placement.allocate_kv_caches``                MorphServe/worker/model.py:187-190 (the K and V pool allocation)
 * ``vmm_pool.VmmKVPool``                             the same pool as ONE tensor over HIP virtual memory
 * ``worker.swap.KVSwapper``                          MorphServe/worker/model.py:468-534 (sequence eviction)
 * ``server.Scheduler``                               MorphServe/server/scheduler.py
@@ -31,6 +32,7 @@ from .worker.kernels.prefill_attn import prefill_attention, chunked_prefill_atte
 from .worker.kernels.rotary_emb import (rotary_embedding_and_store_kvcache, rotary_embedding_inplace,  # noqa: F401
                                         rotary_tables)
 from .elastic_pool import ElasticKVPool  # noqa: F401
+from .kv_placement import allocate_kv_caches  # noqa: F401
 from .vmm_pool import VmmKVPool  # noqa: F401
 from .worker.swap import KVSwapper  # noqa: F401
 from . import swiftllm_c  # noqa: F401
