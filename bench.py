@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes", "placement_probe", "timeline"])
+                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -1464,6 +1464,59 @@ def bench_copy_calibration(args):
 
 
 # ---------------------------------------------------------------------------------
+def bench_layer_handover(args):
+    """A replaced layer's memory becoming pool blocks and going back (config-2 geometry: 1 MiB per block and
+    tensor): ``VmmKVPool.expand_from`` / ``shrink_into`` against ``expand`` / ``shrink_to``, which allocate and
+    free the same amount through the driver.  Llama-3-8B layer: 436 MB in fp16, 116 MB as its 4-bit twin."""
+    import time
+    import torch
+    from morphserve_amd import LayerArena, VmmKVPool
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, HKV, B, D = 32, 8, 16, 128
+    org = args.pool_blocks or 8192
+    layer_bytes, quant_bytes = 436_207_616, 116_000_000
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    by_chunk = {}
+    for cb in (16, 32, 64):
+        pool = VmmKVPool(org, org + 4096, L, HKV, B, D, max_seqs_in_block_table=64, max_blocks_per_seq=128, chunk_blocks=cb)
+        chunk = cb * pool.block_bytes
+        layer = LayerArena(layer_bytes, chunk)
+        n = pool.blocks_available_from(layer, quant_bytes)
+        rows = {"hand_over_in_ms": [], "hand_over_back_ms": [], "allocate_ms": [], "free_ms": []}
+        for it in range(args.warmup + args.steps):
+            a = timed(lambda: pool.expand_from(layer, quant_bytes))
+            assert pool.num_blocks == org + n
+            b = timed(lambda: pool.shrink_into(layer, org))
+            c = timed(lambda: pool.expand(n))
+            d = timed(lambda: pool.shrink_to(org))
+            if it >= args.warmup:
+                for k, v in zip(rows, (a, b, c, d)):
+                    rows[k].append(v)
+        by_chunk[f"{chunk >> 20} MiB"] = {"new_blocks": n, "chunks_moved": 2 * n // cb,
+                                          **{k: round(sorted(v)[len(v) // 2], 3) for k, v in rows.items()}}
+        layer.close()
+        pool.close()
+    best = by_chunk["64 MiB"]
+    return {
+        "metric": "pool growth out of a replaced layer's memory and back, ms per hand-over, 1 MI355X",
+        "value": best["hand_over_in_ms"], "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": best["hand_over_in_ms"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"layer_handover: layer {layer_bytes} B, quantized twin {quant_bytes} B, pool of {org} "
+                               "blocks of 2 MiB (K+V), chunks of 64 MiB; empty tail on the way back"},
+        "by_chunk_size": by_chunk, "zero_fill_included": True, "roofline": None,
+    }
+
+
 def bench_eviction(args):
     """Swap sequences out to host swap space and back (config-2 block geometry, 2 MiB per
     block): whole ``_swap`` calls -- block-manager work, copy, synchronisation -- as PCIe GB/s."""
@@ -1556,7 +1609,7 @@ def main():
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
              "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
              "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving,
-             "timeline": bench_timeline}
+             "timeline": bench_timeline, "layer_handover": bench_layer_handover}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
         # the second target of the path in the same process and the same JSON line: the decode pool is gone

@@ -312,6 +312,18 @@ int mkv_arena_info(const mkv_arena* arena, void** base, uint64_t* reserved_bytes
                    uint64_t* chunk_bytes, uint64_t* mapped_bytes);
 int mkv_arena_resize(mkv_arena* arena, uint64_t mapped_bytes);
 int mkv_arena_destroy(mkv_arena* arena);
+/* The reference's pool grows out of the memory a replaced layer no longer needs
+ * (the bytes of org_range beyond the quantized copy, CS/memory_manager.cpp:69-97)
+ * and that memory serves the restored layer again afterwards
+ * (replace_layer_quant2org after free_kv_cache_tensors, MS/server/memory_utils.py:630-635).
+ * With arenas the same hand-over moves physical chunks: the last `bytes` mapped in
+ * `from` are unmapped there and mapped at the end of `to` -- no allocation, no
+ * free, no copy; the chunks keep their contents (the receiver clears what it
+ * needs cleared).  Same chunk size and device for both; host call, the caller
+ * makes sure no kernel still uses the moved range.  On a failed mapping the
+ * chunk in hand returns to `from`, chunks already moved stay in `to`
+ * (mkv_arena_info tells how far it got). */
+int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes);
 
 /* ---- rotary embedding, optionally fused with the append --------------------- */
 /* rotary_embedding_inplace, MS/worker/kernels/rotary_emb.py:7-58: q [T, Hq, D] and

@@ -13,7 +13,8 @@ Drop-in names (reference file each mirrors):
 * ``swiftllm_c``                                     csrc/src/entrypoints.cpp (KV entries only)
 * ``elastic_pool.ElasticKVPool``                     pool expand / shrink with live-block migration
 * ``kv_placement.allocate_kv_caches``                MorphServe/worker/model.py:187-190 (the K and V pool allocation)
-* ``vmm_pool.VmmKVPool``                             the same pool as ONE tensor over HIP virtual memory
+* ``vmm_pool.VmmKVPool``, ``vmm_pool.LayerArena``      the same pool as ONE tensor over HIP virtual memory; a layer's
+                                                     memory moving into it and back (csrc/src/memory_manager.cpp:69-176)
 * ``worker.swap.KVSwapper``                          MorphServe/worker/model.py:468-534 (sequence eviction)
 * ``server.Scheduler``                               MorphServe/server/scheduler.py
 
@@ -33,6 +34,6 @@ from .worker.kernels.rotary_emb import (rotary_embedding_and_store_kvcache, rota
                                         rotary_tables)
 from .elastic_pool import ElasticKVPool  # noqa: F401
 from .kv_placement import allocate_kv_caches  # noqa: F401
-from .vmm_pool import VmmKVPool  # noqa: F401
+from .vmm_pool import LayerArena, VmmKVPool  # noqa: F401
 from .worker.swap import KVSwapper  # noqa: F401
 from . import swiftllm_c  # noqa: F401

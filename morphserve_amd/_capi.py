@@ -80,6 +80,7 @@ PROTOTYPES = {
     "mkv_arena_info": [_P, C.POINTER(_P), C.POINTER(_U64), C.POINTER(_U64), C.POINTER(_U64)],
     "mkv_arena_resize": [_P, _U64],
     "mkv_arena_destroy": [_P],
+    "mkv_arena_move_tail": [_P, _P, _U64],
     "mkv_rope_store_kvcache": [_P, _P, _P, _P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32,
                                _I32, _I32, _I32, _P],
     "mkv_swap_blocks": [_P, _P, _I64, _I32, _PP, _P, _P, C.POINTER(_I64), _P],

@@ -40,6 +40,22 @@ static int arena_map_one(mkv_arena* a) {
     return MKV_OK;
 }
 
+static int arena_map_handle(mkv_arena* a, hipMemGenericAllocationHandle_t h) {
+    char* at = a->base + a->chunks.size() * a->chunk;
+    MKV_HIP(hipMemMap(at, a->chunk, 0, h, 0));
+    hipMemAccessDesc acc = {};
+    acc.location.type = hipMemLocationTypeDevice;
+    acc.location.id = a->device;
+    acc.flags = hipMemAccessFlagsProtReadWrite;
+    hipError_t e = hipMemSetAccess(at, a->chunk, &acc, 1);
+    if (e != hipSuccess) {
+        (void)hipMemUnmap(at, a->chunk);
+        MKV_HIP(e);
+    }
+    a->chunks.push_back(h);
+    return MKV_OK;
+}
+
 static int arena_unmap_one(mkv_arena* a) {
     char* at = a->base + (a->chunks.size() - 1) * a->chunk;
     MKV_HIP(hipMemUnmap(at, a->chunk));
@@ -106,6 +122,28 @@ int mkv_arena_resize(mkv_arena* arena, uint64_t mapped_bytes) {
     while (arena->chunks.size() > want) {
         int rc = mkv::arena_unmap_one(arena);
         if (rc) return rc;
+    }
+    return MKV_OK;
+}
+
+int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes) {
+    MKV_REQUIRE(from != nullptr && to != nullptr && from != to, "two different arenas are needed");
+    MKV_REQUIRE(from->chunk == to->chunk && from->device == to->device,
+                "both arenas must have the same chunk size and device");
+    MKV_REQUIRE(bytes % from->chunk == 0, "bytes must be a multiple of the chunk size");
+    const size_t n = bytes / from->chunk;
+    MKV_REQUIRE(n <= from->chunks.size(), "the source arena has fewer mapped bytes than that");
+    MKV_REQUIRE((to->chunks.size() + n) * to->chunk <= to->reserved, "the destination's reservation is too small");
+    for (size_t i = 0; i < n; ++i) {
+        hipMemGenericAllocationHandle_t h = from->chunks.back();
+        char* at = from->base + (from->chunks.size() - 1) * from->chunk;
+        MKV_HIP(hipMemUnmap(at, from->chunk));
+        from->chunks.pop_back();
+        int rc = mkv::arena_map_handle(to, h);
+        if (rc) {                                  // put the chunk back where it was; earlier chunks stay moved
+            if (mkv::arena_map_handle(from, h) != MKV_OK) (void)hipMemRelease(h);
+            return rc;
+        }
     }
     return MKV_OK;
 }

@@ -6,7 +6,9 @@ its quantized twin (``org2quant_and_update_kvcache``, :93-116) and shrinks it wh
 the layer is restored (``quant2org_and_update_kvcache``, :617-659).  The weight
 swap itself is not part of this package; where the freed bytes come from is a
 callable ``acquire_segment(layer_id) -> (k_seg, v_seg) | None`` (``None``: let the
-pool allocate a segment of ``seg_blocks`` blocks itself).  Everything else -- the
+pool allocate a segment of ``seg_blocks`` blocks itself) or, for a pool over virtual
+memory, a ``LayerArena`` per replaceable layer whose chunks behind the quantized copy
+move into the pool and back (``layer_arenas``, ``quant_layer_bytes``).  Everything else -- the
 order of the bookkeeping, the layer counters the scheduler reads, the refusal of a
 shrink whose tail segment still holds live blocks -- follows the reference; the
 ``migrate`` switch replaces that refusal by an on-device relocation of the live
@@ -14,7 +16,7 @@ blocks (``ElasticKVPool.shrink_to``).
 """
 from __future__ import annotations
 
-from typing import Callable, List, Optional
+from typing import Callable, Dict, List, Optional
 
 from ..elastic_pool import ElasticKVPool, PoolTooFullError
 
@@ -42,21 +44,43 @@ class PoolEngine:
     functions below: ``.model`` (pool + layer counters), ``.engine_config``, ``.scheduler``."""
 
     def __init__(self, pool: ElasticKVPool, engine_config, num_layers: int, seg_blocks: int,
-                 acquire_segment: Optional[Callable] = None, migrate: bool = True):
+                 acquire_segment: Optional[Callable] = None, migrate: bool = True,
+                 layer_arenas: Optional[Dict[int, object]] = None, quant_layer_bytes: int = 0):
         self.model = _Model(pool, num_layers, seg_blocks)
         self.engine_config = engine_config
         self.acquire_segment = acquire_segment
+        self.layer_arenas = layer_arenas or {}       # layer id -> LayerArena (virtual-memory pools only)
+        self.quant_layer_bytes = quant_layer_bytes   # what the quantized twin keeps at the start of its arena
         self.migrate = migrate
         self.scheduler = None        # set by the owner once the Scheduler exists
         self.migrated_blocks = 0     # live blocks relocated by shrinks so far
+
+
+class _ShrinkInto:
+    """A virtual-memory pool whose ``shrink_to`` hands the memory above the cut to ``arena``."""
+
+    def __init__(self, pool, arena):
+        self._pool, self._arena = pool, arena
+
+    def __getattr__(self, name):
+        return getattr(self._pool, name)
+
+    def shrink_to(self, new_num_blocks: int):
+        return self._pool.shrink_to(new_num_blocks, self._arena)
 
 
 def update_kvcache_after_replacing_layer(engine: PoolEngine, layer_id: int) -> None:
     """memory_utils.py:369-420: append the new segment; ``num_blocks``, ``num_free_blocks``,
     the free map and the scheduler's budget all grow by its block count."""
     model = engine.model
-    seg = engine.acquire_segment(layer_id) if engine.acquire_segment else None
-    if seg is None:
+    arena = engine.layer_arenas.get(layer_id)
+    seg = engine.acquire_segment(layer_id) if engine.acquire_segment and arena is None else None
+    if arena is not None:
+        n = model.pool.expand_from(arena, engine.quant_layer_bytes)
+        if n == 0:                                   # memory_manager.cpp:96-98
+            raise RuntimeError("No space available for new KV cache blocks")
+        model.kv_cache_new_block_size = n
+    elif seg is None:
         model.pool.expand(model.kv_cache_new_block_size)
     else:
         model.pool.expand(int(seg[0].shape[0]), seg[0], seg[1])
@@ -92,6 +116,9 @@ def quant2org_and_update_kvcache(engine: PoolEngine, update_kvcache: bool = True
     if update_kvcache:
         pool = model.pool
         contiguous = hasattr(pool, "tail_unused")          # a virtual-memory pool: no segments to pop
+        arena = engine.layer_arenas.get(layer_id)
+        if arena is not None:                              # the memory goes back to the layer it came from
+            pool = _ShrinkInto(pool, arena)
         if contiguous and pool.tail_unused(model.kv_cache_new_block_size):
             pool.shrink_to(pool.num_blocks - model.kv_cache_new_block_size)
         elif not contiguous and pool.shrink_tail_if_unused():

@@ -90,9 +90,9 @@ def register_layer_memory_quant(layer_id: int, start_addr_int: int, size: int) -
 class _RawDeviceMemory:
     """Non-owning view of device memory for ``torch.as_tensor``."""
 
-    def __init__(self, address: int, shape: Tuple[int, ...], keepalive=None):
+    def __init__(self, address: int, shape: Tuple[int, ...], keepalive=None, typestr: str = "<f2"):
         self.__cuda_array_interface__ = {
-            "shape": tuple(shape), "typestr": "<f2", "data": (int(address), False),
+            "shape": tuple(shape), "typestr": typestr, "data": (int(address), False),
             "version": 2, "strides": None,
         }
         self._keepalive = keepalive

@@ -42,10 +42,47 @@ class _Arena:
         _capi.check(_capi.lib().mkv_arena_info(self.handle, None, None, None, C.byref(n)))
         return int(n.value)
 
+    def move_tail_to(self, other: "_Arena", nbytes: int) -> None:
+        """Hand the physical memory behind the last ``nbytes`` mapped here over to the end of ``other``."""
+        _capi.check(_capi.lib().mkv_arena_move_tail(self.handle, other.handle, nbytes))
+
     def close(self) -> None:
         if self.handle:
             _capi.check(_capi.lib().mkv_arena_destroy(self.handle))
             self.handle = C.c_void_p()
+
+
+class LayerArena(_Arena):
+    """Device memory of one replaceable transformer layer, in chunks a ``VmmKVPool`` can take over.
+
+    The reference keeps a layer's fp16 weights in one range, copies the quantized twin to the START of that
+    range when the layer is replaced and turns the rest into KV tensors (csrc/src/memory_manager.cpp:69-176);
+    restoring the layer copies the fp16 weights back from the host (memory_utils.py:635).  Here the range is
+    an arena of ``nbytes`` rounded up to whole chunks, all mapped; ``VmmKVPool.expand_from`` moves the chunks
+    behind ``keep_bytes`` to the end of the pool and ``VmmKVPool.shrink_into`` brings them back."""
+
+    def __init__(self, nbytes: int, chunk_bytes: int, device: str = "cuda"):
+        self.chunk_bytes = chunk_bytes
+        self.capacity = -(-nbytes // chunk_bytes) * chunk_bytes
+        super().__init__(self.capacity, chunk_bytes)
+        self.device = torch.device(device, torch.cuda.current_device()) if device == "cuda" else torch.device(device)
+        try:
+            self.resize(self.capacity)
+        except Exception:
+            self.close()
+            raise
+
+    def tensor(self, offset_bytes: int, shape, dtype=torch.float16) -> torch.Tensor:
+        """A tensor over ``[offset_bytes, offset_bytes + size)`` of the arena; the range must be mapped for
+        as long as the tensor is used."""
+        shape = tuple(int(x) for x in shape)
+        nbytes = torch.empty((), dtype=dtype).element_size()
+        for x in shape:
+            nbytes *= x
+        if offset_bytes < 0 or offset_bytes + nbytes > self.mapped_bytes():
+            raise ValueError(f"[{offset_bytes}, {offset_bytes + nbytes}) is outside the {self.mapped_bytes()} mapped bytes")
+        typestr = {torch.float16: "<f2", torch.uint8: "|u1", torch.int32: "<i4", torch.float32: "<f4"}[dtype]
+        return torch.as_tensor(_RawDeviceMemory(self.base + offset_bytes, shape, self, typestr), device=self.device)
 
 
 class VmmKVPool(ElasticKVPool):
@@ -81,6 +118,9 @@ class VmmKVPool(ElasticKVPool):
         except Exception:
             self._k_arena.resize(self._v_arena.mapped_bytes())
             raise
+        self._make_views(num_blocks)
+
+    def _make_views(self, num_blocks: int) -> None:
         shape = (num_blocks, *self.shape_tail)
         self.k_cache = torch.as_tensor(_RawDeviceMemory(self._k_arena.base, shape, self._k_arena), device=self.device)
         self.v_cache = torch.as_tensor(_RawDeviceMemory(self._v_arena.base, shape, self._v_arena), device=self.device)
@@ -103,8 +143,12 @@ class VmmKVPool(ElasticKVPool):
             raise ValueError(f"the pool grows in multiples of {self.chunk_blocks} blocks")
         if bm.num_blocks + num_new_blocks > self.max_blocks:
             raise ValueError(f"at most {self.max_blocks} blocks were reserved")
+        self._map(bm.num_blocks + num_new_blocks)
+        self._grew_by(num_new_blocks)
+
+    def _grew_by(self, num_new_blocks: int) -> None:
+        bm = self.block_manager
         old = bm.num_blocks
-        self._map(old + num_new_blocks)
         self._zero(old, num_new_blocks)
         bm.num_blocks += num_new_blocks
         bm.num_free_blocks += num_new_blocks
@@ -113,6 +157,45 @@ class VmmKVPool(ElasticKVPool):
         new_map[old:] = True
         bm.is_block_free = new_map
 
+    def blocks_available_from(self, donor: "LayerArena", keep_bytes: int) -> int:
+        """How many blocks ``expand_from(donor, keep_bytes)`` would add: the donor's mapped chunks behind
+        ``keep_bytes`` split evenly between K and V, capped by the reservation."""
+        if donor.chunk_bytes != self.chunk_blocks * self.block_bytes:
+            raise ValueError("the donor's chunks must have the pool's chunk size")
+        keep_chunks = -(-keep_bytes // donor.chunk_bytes)
+        free_chunks = donor.mapped_bytes() // donor.chunk_bytes - keep_chunks
+        room = (self.max_blocks - self.block_manager.num_blocks) // self.chunk_blocks
+        return max(0, min(free_chunks // 2, room)) * self.chunk_blocks
+
+    def expand_from(self, donor: "LayerArena", keep_bytes: int) -> int:
+        """Grow by the memory ``donor`` no longer needs once its first ``keep_bytes`` hold the quantized
+        layer (``acquire_new_kvcache``, csrc/src/memory_manager.cpp:69-176, followed by
+        ``update_kvcache_after_replacing_layer``, memory_utils.py:369-420): the donor's chunks behind
+        ``keep_bytes`` move to the end of K and of V (half each), are zero filled and join the free map.
+        Nothing is allocated or copied.  Returns the number of new blocks (0: nothing to take)."""
+        n = self.blocks_available_from(donor, keep_bytes)
+        if n == 0:
+            return 0
+        nbytes = n * self.block_bytes
+        torch.cuda.synchronize(self.device)                          # nothing may still use the donor's tail
+        self.k_cache = self.v_cache = None
+        donor.move_tail_to(self._k_arena, nbytes)
+        try:
+            donor.move_tail_to(self._v_arena, nbytes)
+        except Exception:
+            moved = self._k_arena.mapped_bytes() - self.block_manager.num_blocks * self.block_bytes
+            self._k_arena.move_tail_to(donor, moved)
+            self._make_views(self.block_manager.num_blocks)
+            raise
+        self._make_views(self.block_manager.num_blocks + n)
+        self._grew_by(n)
+        return n
+
+    def shrink_into(self, donor: "LayerArena", new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """``shrink_to(new_num_blocks)`` with the memory above the cut handed back to ``donor`` instead of
+        the driver (the restored layer's weights are copied there next, memory_utils.py:635)."""
+        return self.shrink_to(new_num_blocks, donor)
+
     def tail_unused(self, num_blocks: int) -> bool:
         """True when none of the last ``num_blocks`` blocks is live."""
         bm = self.block_manager
@@ -120,11 +203,17 @@ class VmmKVPool(ElasticKVPool):
                                                   bm.num_blocks, self._result.data_ptr(), _capi.current_stream()))
         return int(self._result[0].item()) == 0
 
-    def shrink_to(self, new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    def shrink_to(self, new_num_blocks: int, donor: "LayerArena" = None) -> Tuple[torch.Tensor, torch.Tensor]:
         """Shrink to ``new_num_blocks``: live blocks above the cut move to the lowest free ids
-        below it, the block table is rewritten, the memory above the cut is unmapped.
+        below it, the block table is rewritten, the memory above the cut is unmapped (or, with a
+        ``donor``, mapped back at the end of that arena).
         Returns the move lists; raises ``RuntimeError`` (state untouched) when they do not fit."""
         bm = self.block_manager
+        if donor is not None:
+            if donor.chunk_bytes != self.chunk_blocks * self.block_bytes:
+                raise ValueError("the donor's chunks must have the pool's chunk size")
+            if donor.mapped_bytes() + 2 * (bm.num_blocks - new_num_blocks) * self.block_bytes > donor.capacity:
+                raise ValueError("the donor has no room for that many chunks")
         if not 0 < new_num_blocks <= bm.num_blocks or new_num_blocks % self.chunk_blocks:
             raise ValueError(f"new size {new_num_blocks} must be a positive multiple of {self.chunk_blocks} "
                              f"and at most {bm.num_blocks}")
@@ -137,7 +226,13 @@ class VmmKVPool(ElasticKVPool):
         bm.num_free_blocks -= removed
         bm.is_block_free = bm.is_block_free[:new_num_blocks].clone()
         torch.cuda.synchronize(self.device)                          # nothing may still read the tail
-        self._map(new_num_blocks)
+        if donor is None:
+            self._map(new_num_blocks)
+        else:
+            self.k_cache = self.v_cache = None
+            self._v_arena.move_tail_to(donor, removed * self.block_bytes)
+            self._k_arena.move_tail_to(donor, removed * self.block_bytes)
+            self._make_views(new_num_blocks)
         return src, dst
 
     # the segment-based entry points of the parent do not apply

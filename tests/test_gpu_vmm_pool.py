@@ -188,3 +188,153 @@ def test_eviction_on_a_virtual_memory_pool(cuda):
         assert np.array_equal(bits(pool.v_cache).reshape(-1), arena[32 * blk:].view(np.uint16))
     finally:
         pool.close()
+
+
+# ---- a layer's memory moving into the pool and back ---------------------------------------------------------
+def _free_device_bytes():
+    torch.cuda.synchronize()
+    return torch.cuda.mem_get_info()[0]
+
+
+def test_pool_grows_out_of_a_replaced_layers_memory_and_gives_it_back(cuda):
+    """``acquire_new_kvcache`` (csrc/src/memory_manager.cpp:69-176) over virtual memory: the chunks of a
+    layer's arena behind the quantized copy become pool blocks (zero filled, free), the quantized bytes at
+    the start of the arena and every old pool byte stay as they were, no device memory is allocated or
+    freed on the way, and ``shrink_into`` (with live blocks above the cut) returns the memory to the layer."""
+    from morphserve_amd import LayerArena
+    cb, org = 64, 64
+    pool = VmmKVPool(org, 256, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=32, chunk_blocks=cb)
+    chunk = cb * pool.block_bytes                      # 1 MiB
+    layer_bytes = 9 * chunk - 1000                     # fp16 layer: 9 chunks (the last one partly used)
+    quant_bytes = 2 * chunk + 6                        # its quantized twin: needs 3 chunks
+    layer = LayerArena(layer_bytes, chunk)
+    try:
+        rng = np.random.default_rng(5)
+        blk = L * HKV * B * D
+        mapped = lambda: layer.mapped_bytes() + pool._k_arena.mapped_bytes() + pool._v_arena.mapped_bytes()
+        assert layer.capacity == 9 * chunk and layer.mapped_bytes() == 9 * chunk
+        w = layer.tensor(0, (layer_bytes // 2,), torch.float16)
+        w.copy_(torch.from_numpy(rng.standard_normal(layer_bytes // 2, dtype=np.float32).astype(np.float16)))
+        head = bits(layer.tensor(0, (quant_bytes // 2,), torch.float16))
+        arena = _mirror(pool, org, rng)
+        k_addr, v_addr = pool.k_cache.data_ptr(), pool.v_cache.data_ptr()
+        ob = R.BlockManagerOracle("GPU", org, 8, 32, B)
+        total_mapped, free_before = mapped(), _free_device_bytes()
+
+        assert pool.blocks_available_from(layer, quant_bytes) == 3 * cb              # (9 - 3) // 2 chunks each
+        n = pool.expand_from(layer, quant_bytes)
+        ob.expand(n)
+        assert n == 192 and pool.num_blocks == 256 and layer.mapped_bytes() == 3 * chunk
+        assert mapped() == total_mapped and abs(_free_device_bytes() - free_before) < 4 * chunk   # 6 chunks moved
+        assert pool.k_cache.data_ptr() == k_addr and pool.v_cache.data_ptr() == v_addr
+        assert np.array_equal(bits(pool.k_cache[:org]).reshape(-1), arena[:org * blk].view(np.uint16))
+        assert np.array_equal(bits(pool.v_cache[:org]).reshape(-1), arena[org * blk:].view(np.uint16))
+        assert not pool.k_cache[org:].any() and not pool.v_cache[org:].any()         # the old weights are gone
+        assert_state_equal(manager_state(pool.block_manager), ob.snapshot(), "grown out of the layer")
+        assert np.array_equal(bits(layer.tensor(0, (quant_bytes // 2,), torch.float16)), head)   # the twin is untouched
+        with pytest.raises(ValueError):
+            layer.tensor(3 * chunk, (16,), torch.float16)                             # no longer the layer's
+
+        # sequences that live in the new blocks; then the layer comes back and they move below the cut
+        bm = pool.block_manager
+        lens = [16 * 30, 16 * 30, 16 * 25, 16 * 9, 40]
+        ids = list(range(len(lens)))
+        bm.allocate_blocks_for_seqs(_i32(ids, cuda), _i32(lens, cuda))
+        ob.allocate_blocks_for_seqs(np.array(ids), np.array(lens))
+        bm.free_blocks_for_seqs(_i32([0, 1], cuda))
+        ob.free_blocks_for_seqs(np.array([0, 1]))
+        lens2 = [16 * 12, 16 * 3]
+        bm.allocate_blocks_for_seqs(_i32([5, 6], cuda), _i32(lens2, cuda))
+        ob.allocate_blocks_for_seqs(np.array([5, 6]), np.array(lens2))
+        total = pool.num_blocks
+        full = _mirror(pool, total, rng)
+        lay = R.plain_layout(total, L, HKV, B, D)
+        want_src, want_dst = R.apply_migration(full, lay, ob, org)
+        src, dst = pool.shrink_into(layer, org)
+        assert len(want_src) > 0 and src.cpu().tolist() == want_src.tolist() and dst.cpu().tolist() == want_dst.tolist()
+        assert_state_equal(manager_state(bm), ob.snapshot(), "after the layer came back")
+        assert np.array_equal(bits(pool.k_cache).reshape(-1), full[:org * blk].view(np.uint16))
+        assert np.array_equal(bits(pool.v_cache).reshape(-1), full[total * blk:(total + org) * blk].view(np.uint16))
+        assert layer.mapped_bytes() == 9 * chunk and mapped() == total_mapped
+        assert abs(_free_device_bytes() - free_before) < 4 * chunk
+        assert np.array_equal(bits(layer.tensor(0, (quant_bytes // 2,), torch.float16)), head)
+        w = layer.tensor(0, (layer_bytes // 2,), torch.float16)                      # the restored weights fit again
+        w.fill_(1.5)
+        assert float(w.min()) == 1.5 and pool.k_cache.data_ptr() == k_addr
+        assert np.array_equal(bits(pool.k_cache).reshape(-1), full[:org * blk].view(np.uint16))
+    finally:
+        layer.close()
+        pool.close()
+
+
+def test_hand_over_limits(cuda):
+    from morphserve_amd import LayerArena, _capi
+    pool = VmmKVPool(32, 64, L, HKV, B, D, max_seqs_in_block_table=4, max_blocks_per_seq=16, chunk_blocks=16)
+    chunk = 16 * pool.block_bytes
+    layer = LayerArena(10 * chunk, chunk)
+    other = LayerArena(chunk, 2 * chunk)
+    try:
+        assert pool.blocks_available_from(layer, 0) == 32           # capped by the reservation (64 - 32 blocks)
+        with pytest.raises(ValueError):
+            pool.blocks_available_from(other, 0)                     # another chunk size
+        assert pool.expand_from(layer, 10 * chunk) == 0 and pool.num_blocks == 32   # the twin needs it all
+        assert pool.expand_from(layer, 9 * chunk) == 0               # one spare chunk cannot serve K and V
+        assert pool.expand_from(layer, 0) == 32 and layer.mapped_bytes() == 6 * chunk
+        with pytest.raises(ValueError):
+            pool.shrink_to(48, other)
+        lib = _capi.lib()
+        assert lib.mkv_arena_move_tail(layer.handle, layer.handle, chunk) == _capi.MKV_EINVAL
+        assert lib.mkv_arena_move_tail(layer.handle, other.handle, 2 * chunk) == _capi.MKV_EINVAL   # chunk sizes differ
+        assert lib.mkv_arena_move_tail(layer.handle, pool._k_arena.handle, chunk) == _capi.MKV_EINVAL  # reservation full
+        assert lib.mkv_arena_move_tail(layer.handle, pool._k_arena.handle, chunk // 2) == _capi.MKV_EINVAL
+        pool.shrink_into(layer, 32)
+        assert layer.mapped_bytes() == 10 * chunk
+        with pytest.raises(ValueError):
+            pool.shrink_into(layer, 16)                              # the layer's arena is complete already
+    finally:
+        other.close()
+        layer.close()
+        pool.close()
+
+
+def test_layer_replacement_bookkeeping_over_layer_arenas(cuda):
+    """``org2quant_and_update_kvcache`` / ``quant2org_and_update_kvcache`` (memory_utils.py:93-116, :617-659)
+    with the pool's growth coming out of each replaced layer's own arena and going back into it."""
+    from morphserve_amd import LayerArena
+    from morphserve_amd.server.memory_utils import (PoolEngine, org2quant_and_update_kvcache,
+                                                    quant2org_and_update_kvcache)
+    cb = 16
+    pool = VmmKVPool(32, 32 + 2 * 48, L, HKV, B, D, max_seqs_in_block_table=4, max_blocks_per_seq=64, chunk_blocks=cb)
+    chunk = cb * pool.block_bytes
+    arenas = {0: LayerArena(8 * chunk, chunk), 1: LayerArena(8 * chunk, chunk)}
+    try:
+        eng = PoolEngine(pool, None, num_layers=2, seg_blocks=0, layer_arenas=arenas, quant_layer_bytes=2 * chunk - 7)
+        org2quant_and_update_kvcache(eng)                                  # the last layer goes first (model.py:81)
+        assert pool.num_blocks == 80 and arenas[1].mapped_bytes() == 2 * chunk and arenas[0].mapped_bytes() == 8 * chunk
+        assert eng.model.kv_cache_new_block_size == 48 and eng.model.layer_quant_list == [1]
+        org2quant_and_update_kvcache(eng)
+        assert pool.num_blocks == 128 and arenas[0].mapped_bytes() == 2 * chunk
+        with pytest.raises(RuntimeError):
+            org2quant_and_update_kvcache(eng)                              # no layer left
+        bm = pool.block_manager
+        bm.allocate_blocks_for_seqs(_i32([0, 1], cuda), _i32([16 * 60, 16 * 50], cuda))      # blocks 0..109
+        bm.free_blocks_for_seqs(_i32([0], cuda))                                              # 60..109 stay live
+        mark = torch.arange(128, dtype=torch.float16, device=cuda).view(128, 1, 1, 1, 1)
+        pool.k_cache.copy_(mark.expand_as(pool.k_cache))
+        pool.v_cache.copy_((-mark).expand_as(pool.v_cache))
+        row_before = bm.block_table[1, :50].cpu().tolist()
+        assert quant2org_and_update_kvcache(eng) is True                   # layer 0 comes back: cut at 80
+        assert pool.num_blocks == 80 and arenas[0].mapped_bytes() == 8 * chunk and eng.migrated_blocks == 30
+        row = bm.block_table[1, :50].cpu().tolist()
+        assert row_before == list(range(60, 110)) and row[:20] == list(range(60, 80)) and row[20:] == list(range(30))
+        assert pool.k_cache[row, 0, 0, 0, 0].cpu().tolist() == [float(x) for x in range(60, 110)]
+        assert pool.v_cache[row, 1, 1, 15, 127].cpu().tolist() == [-float(x) for x in range(60, 110)]
+        assert quant2org_and_update_kvcache(eng) is False                  # 50 live blocks do not fit in 32
+        assert pool.num_blocks == 80 and arenas[1].mapped_bytes() == 2 * chunk
+        bm.free_blocks_for_seqs(_i32([1], cuda))
+        assert quant2org_and_update_kvcache(eng) is True
+        assert pool.num_blocks == 32 and arenas[1].mapped_bytes() == 8 * chunk and eng.model.layer_quant_list == []
+    finally:
+        for a in arenas.values():
+            a.close()
+        pool.close()
