@@ -81,7 +81,10 @@ class LayerArena(_Arena):
             nbytes *= x
         if offset_bytes < 0 or offset_bytes + nbytes > self.mapped_bytes():
             raise ValueError(f"[{offset_bytes}, {offset_bytes + nbytes}) is outside the {self.mapped_bytes()} mapped bytes")
-        typestr = {torch.float16: "<f2", torch.uint8: "|u1", torch.int32: "<i4", torch.float32: "<f4"}[dtype]
+        typestrs = {torch.float16: "<f2", torch.uint8: "|u1", torch.int8: "|i1", torch.int32: "<i4", torch.float32: "<f4"}
+        if dtype not in typestrs:
+            raise ValueError(f"{dtype}: take a uint8 tensor and .view() it")
+        typestr = typestrs[dtype]
         return torch.as_tensor(_RawDeviceMemory(self.base + offset_bytes, shape, self, typestr), device=self.device)
 
 
