@@ -35,6 +35,20 @@ class LlamaModelConfig:
         """Bytes of one pool block, K and V together."""
         return block_size * self.get_kvslot_size(dtype)
 
+    def num_blocks_that_fit(self, block_size: int, free_memory: int, total_memory: int,
+                            gpu_mem_utilization: float, dtype: torch.dtype = torch.float16) -> int:
+        """The pool size ``LlamaModel.profile_num_blocks`` arrives at once its forged prefill batch has run
+        (MorphServe/worker/model.py:161-171): with ``free_memory, total_memory`` as ``torch.cuda.mem_get_info``
+        reports them at the peak, ``floor((total * utilization - (total - free)) / block bytes)``;
+        ``RuntimeError`` when the peak already exceeds the usable share."""
+        peak = total_memory - free_memory
+        usable = total_memory * gpu_mem_utilization
+        if usable < peak:
+            gb = 1024 ** 3
+            raise RuntimeError(f"Peak memory {peak / gb:.2f} GB exceeds usable memory {usable / gb:.2f} GB "
+                               f"({total_memory / gb:.2f} GB * {gpu_mem_utilization})")
+        return int((usable - peak) // self.get_block_bytes(block_size, dtype))
+
     @staticmethod
     def load_from_model_path(model_path: str) -> "LlamaModelConfig":
         with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:

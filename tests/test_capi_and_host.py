@@ -217,6 +217,15 @@ def test_model_config_kv_sizes_known_answers(tmp_path):
         assert cfg.get_kvslot_size() == slot, name
         assert cfg.get_kvslot_size(torch.float32) == 2 * slot, name
         assert cfg.get_block_bytes(16) == block, name
+    # pool sizing (MorphServe/worker/model.py:161-171), worked by hand: a 288 GiB card at 0.9 with 30 GiB in use at
+    # the peak leaves 229.2 GiB = 117 350.4 blocks of 2 MiB; 48 GiB of 64 GiB at 0.8 leaves 3.2 GiB = 1638.4 blocks
+    gib = 1 << 30
+    cfg8 = LlamaModelConfig(dict(shapes["llama-3-8b"][0], model_type="llama"))
+    assert cfg8.num_blocks_that_fit(16, 258 * gib, 288 * gib, 0.9) == 117350
+    assert cfg8.num_blocks_that_fit(16, 16 * gib, 64 * gib, 0.8) == 1638
+    assert cfg8.num_blocks_that_fit(16, 16 * gib, 64 * gib, 0.75) == 0
+    with pytest.raises(RuntimeError, match="exceeds usable memory"):
+        cfg8.num_blocks_that_fit(16, 16 * gib, 64 * gib, 0.7)
     d = tmp_path / "m"
     d.mkdir()
     (d / "config.json").write_text(json.dumps(dict(shapes["llama-3-8b"][0], model_type="llama", rope_scaling=None)))
