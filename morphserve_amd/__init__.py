@@ -15,6 +15,7 @@ Drop-in names (reference file each mirrors):
 * ``kv_placement.allocate_kv_caches``                MorphServe/worker/model.py:187-190 (the K and V pool allocation)
 * ``vmm_pool.VmmKVPool``, ``vmm_pool.LayerArena``      the same pool as ONE tensor over HIP virtual memory; a layer's
                                                      memory moving into it and back (csrc/src/memory_manager.cpp:69-176)
+* ``worker.layers.attention_section``                MorphServe/worker/layers/transformer_layer.py:93-191 (rotary .. decode attention)
 * ``worker.swap.KVSwapper``                          MorphServe/worker/model.py:468-534 (sequence eviction)
 * ``server.Scheduler``                               MorphServe/server/scheduler.py
 
@@ -36,4 +37,5 @@ from .elastic_pool import ElasticKVPool  # noqa: F401
 from .kv_placement import allocate_kv_caches  # noqa: F401
 from .vmm_pool import LayerArena, VmmKVPool  # noqa: F401
 from .worker.swap import KVSwapper  # noqa: F401
+from .worker.layers import attention_section  # noqa: F401
 from . import swiftllm_c  # noqa: F401
