@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover"])
+                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover", "step_state"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -1464,6 +1464,59 @@ def bench_copy_calibration(args):
 
 
 # ---------------------------------------------------------------------------------
+def bench_step_state(args):
+    """Host time of a step's preparation (MorphServe/worker/model.py:318-436): the reference's way -- one device
+    tensor per host list, an arange per prefill sequence, two gathers -- against ``StepStateBuilder`` (one pinned
+    staging buffer, one asynchronous copy, two gathers), block allocation excluded from both."""
+    import torch
+    from morphserve_amd import StepStateBuilder, build_infer_state
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    rng = np.random.default_rng(args.seed)
+    cos = torch.randn((4096 + 128, 64), dtype=torch.float16, device=dev)
+    sin = torch.randn_like(cos)
+    builder = StepStateBuilder(256, 16384, 8, 128, cos_cached=cos, sin_cached=sin)
+
+    def reference_way(p, ids, d):
+        st = build_infer_state(p, ids, d, 8, 128)
+        pos = torch.cat((
+            torch.concat([torch.arange(0, x, device=dev, dtype=torch.int32) for x in p])
+            if p else torch.empty(0, device=dev, dtype=torch.int32), st.decoding_seq_lens - 1), dim=0)
+        st.position_cos, st.position_sin = cos[pos], sin[pos]
+        return st
+
+    shapes = {"cfg2 decode step (64 decoding)": ([], rng.integers(1024, 1537, size=64).tolist()),
+              "cfg4 mixed step (8 x 512 prefill + 120 decoding)": ([512] * 8, rng.integers(16, 769, size=120).tolist()),
+              "cfg5 decode step (128 decoding)": ([], rng.integers(1024, 1537, size=128).tolist())}
+    out = {}
+    for name, (p, d) in shapes.items():
+        ids = list(range(len(p) + len(d)))
+        row = {}
+        for label, fn in (("one_tensor_per_list_us", reference_way), ("one_staging_copy_us", builder.build)):
+            for _ in range(max(args.warmup, 3)):
+                fn(p, ids, d)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps * 5):
+                fn(p, ids, d)
+            host = (time.perf_counter() - t0) / (args.steps * 5) * 1e6       # until the calls return
+            torch.cuda.synchronize()
+            row[label] = round(host, 1)
+        a, b = reference_way(p, ids, d), builder.build(p, ids, d)
+        assert torch.equal(a.position_cos, b.position_cos) and torch.equal(a.seq_ids, b.seq_ids)
+        out[name] = row
+    first = out["cfg2 decode step (64 decoding)"]
+    return {
+        "metric": "host time to prepare one step's LlamaInferState (lists -> device tensors, positions, rotary rows)",
+        "value": first["one_staging_copy_us"], "unit": "us", "n_gpus": 1, "steps": args.steps * 5, "warmup": args.warmup,
+        "ms_per_step": round(first["one_staging_copy_us"] / 1e3, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+        "config": {"workload": "step_state: the preparation of model.py:318-436 for three batch shapes"},
+        "shapes": out, "roofline": None,
+    }
+
+
 def bench_layer_handover(args):
     """A replaced layer's memory becoming pool blocks and going back (config-2 geometry: 1 MiB per block and
     tensor): ``VmmKVPool.expand_from`` / ``shrink_into`` against ``expand`` / ``shrink_to``, which allocate and
@@ -1609,7 +1662,7 @@ def main():
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
              "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
              "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving,
-             "timeline": bench_timeline, "layer_handover": bench_layer_handover}
+             "timeline": bench_timeline, "layer_handover": bench_layer_handover, "step_state": bench_step_state}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
         # the second target of the path in the same process and the same JSON line: the decode pool is gone

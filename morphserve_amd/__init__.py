@@ -24,7 +24,8 @@ ctypes; nothing here falls back to eager PyTorch.
 """
 from . import _capi  # noqa: F401
 from .model_config import LlamaModelConfig  # noqa: F401
-from .worker.infer_state import LlamaInferState, build_infer_state, select_seq_block_size  # noqa: F401
+from .worker.infer_state import (LlamaInferState, StepStateBuilder, build_infer_state,  # noqa: F401
+                                 select_seq_block_size)
 from .worker.block_manager import BlockManager  # noqa: F401
 from .worker.kernels.kvcache_mgmt import store_kvcache  # noqa: F401
 from .worker.kernels._deferred import enable_deferred_decode_append, flush as flush_pending_appends  # noqa: F401

@@ -233,3 +233,44 @@ def test_model_config_kv_sizes_known_answers(tmp_path):
     assert (cfg.num_layers, cfg.num_q_heads, cfg.num_kv_heads, cfg.rope_scaling) == (32, 32, 8, 1.0)
     with pytest.raises(ValueError):
         LlamaModelConfig(dict(shapes["llama-2-7b"][0], model_type="gpt2"))
+
+
+def test_step_state_builder_matches_the_field_by_field_builder():
+    """One staging buffer instead of one tensor per list (model.py:318-436): every field equal to
+    ``build_infer_state``'s, positions = 0..len-1 per prefill sequence then len-1 per decoding one, over
+    consecutive steps that reuse the buffers."""
+    import numpy as np
+    import torch
+
+    from morphserve_amd import StepStateBuilder, build_infer_state
+    cos = torch.arange(4096, dtype=torch.float32).view(-1, 1).expand(4096, 4).contiguous()
+    b = StepStateBuilder(16, 4096, 8, 128, cos_cached=cos, sin_cached=-cos, device="cpu")
+    rng = np.random.default_rng(0)
+    kept = []
+    for step in range(12):
+        P, n = int(rng.integers(0, 6)), int(rng.integers(0, 8))
+        if P + n == 0:
+            n = 1
+        p = rng.integers(1, 300, size=P).tolist()
+        d = rng.integers(1, 2000, size=n).tolist()
+        ids = rng.permutation(64)[:P + n].tolist()
+        s = b.build(p, ids, d)
+        r = build_infer_state(p, ids, d, 8, 128, device="cpu")
+        for f in ("seq_ids", "prefill_seq_start_locs", "prefill_seq_start_locs_with_end", "prefill_seq_lens",
+                  "decoding_seq_lens"):
+            assert torch.equal(getattr(s, f), getattr(r, f)), (step, f)
+            assert getattr(s, f).dtype == torch.int32
+        for f in ("batch_size", "num_tokens", "num_prefill_seqs", "num_prefill_tokens", "max_prefill_len",
+                  "num_decoding_seqs", "max_decoding_len", "seq_block_size", "num_seq_blocks", "softmax_scale",
+                  "num_blocks_org", "ignore_kvcache"):
+            assert getattr(s, f) == getattr(r, f), (step, f)
+        pos = np.concatenate([np.arange(x) for x in p] + [np.asarray(d, dtype=np.int64) - 1]) if P + n else []
+        assert s.position_cos[:, 0].tolist() == [float(x) for x in pos]
+        assert s.position_sin[:, 3].tolist() == [-float(x) for x in pos]
+        kept.append((s, ids))
+        if len(kept) >= 2:                                   # the state before this one is still intact (two slots)
+            assert kept[-2][0].seq_ids.tolist() == kept[-2][1]
+    with pytest.raises(ValueError):
+        b.build([4000, 200], [0, 1], [])
+    with pytest.raises(ValueError):
+        b.build([], [0, 1], [5])

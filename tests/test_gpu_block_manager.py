@@ -192,3 +192,41 @@ def test_expand_shrink_round_trip(cuda):
     assert_state_equal(manager_state(bm), ob.snapshot(), "refused")
     bm.free_blocks_for_seqs(_i32([1], cuda))
     assert pool.shrink_tail_if_unused()
+
+
+def test_step_state_builder_on_the_device(cuda):
+    """``StepStateBuilder`` (one pinned staging buffer, one asynchronous copy per step) against the field-by-field
+    builder and the block-manager oracle over a run of steps: fields, gathered rotary rows and the allocations
+    of ``model.py:364-368``."""
+    from oracle import rope_cpu as RO
+    from morphserve_amd import BlockManager, StepStateBuilder, build_infer_state
+    ct, st_ = RO.rotary_tables(128, 4096)
+    cos, sin = torch.from_numpy(ct).to(cuda), torch.from_numpy(st_).to(cuda)
+    bm = BlockManager("GPU", 2048, 64, 128, 16, device="cuda")
+    ob = R.BlockManagerOracle("GPU", 2048, 64, 128, 16)
+    b = StepStateBuilder(64, 8192, 8, 128, cos_cached=cos, sin_cached=sin)
+    rng = np.random.default_rng(3)
+    lens = {}
+    for step in range(10):
+        new = [int(x) for x in rng.permutation(64) if int(x) not in lens][:int(rng.integers(0, 4))]
+        p = rng.integers(1, 400, size=len(new)).tolist()
+        running = sorted(lens)
+        d = [lens[s] + 1 for s in running]
+        ids = new + running
+        if not ids:
+            continue
+        s = b.build(p, ids, d, block_manager=bm)
+        r = build_infer_state(p, ids, d, 8, 128)
+        ob.allocate_blocks_for_seqs(np.asarray(ids), np.asarray(p + d))
+        for f in ("seq_ids", "prefill_seq_start_locs", "prefill_seq_start_locs_with_end", "prefill_seq_lens",
+                  "decoding_seq_lens"):
+            assert torch.equal(getattr(s, f), getattr(r, f)), (step, f)
+        assert (s.seq_block_size, s.num_seq_blocks, s.num_blocks_org) == (r.seq_block_size, r.num_seq_blocks, 2048)
+        pos = np.concatenate([np.arange(x) for x in p] + [np.asarray(d, dtype=np.int64) - 1]).astype(np.int64)
+        assert np.array_equal(bits(s.position_cos), ct[pos].view(np.uint16))
+        assert np.array_equal(bits(s.position_sin), st_[pos].view(np.uint16))
+        assert_state_equal(manager_state(bm), ob.snapshot(), f"step {step}")
+        for sid, n in zip(new, p):
+            lens[sid] = n
+        for sid in running:
+            lens[sid] += 1
