@@ -110,3 +110,69 @@ def test_prefill_without_a_cache(cuda):
     want = R.prefill_attention(q, k, v, starts, np.asarray(p_lens), D ** -0.5, math="np32")
     assert np.array_equal(bits(qg), bits(q)) and np.array_equal(bits(kg), bits(k))
     assert_attn_close(o.cpu().numpy().reshape(P, Hq, D), np.asarray(want), "prefill without a cache")
+
+
+def test_serving_steps_with_the_step_builder(cuda):
+    """Several engine steps in a row, each prepared by ``StepStateBuilder`` (lists -> state, positions, rotary rows,
+    block allocation) and run by ``attention_section`` for every layer: prompts arrive, decode, finish and free
+    their blocks.  After every step the pool bytes, the allocator state and ``o`` are checked against the oracle
+    run through the same steps."""
+    from gpu_helpers import assert_state_equal, manager_state
+    from helpers import Cfg
+    from morphserve_amd import ElasticKVPool, StepStateBuilder
+    L, Hq, Hkv, D, B, NB = 2, 8, 2, 128, 16, 96
+    pool = ElasticKVPool(NB, L, Hkv, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=24, device="cuda")
+    bm = pool.block_manager
+    ob = R.BlockManagerOracle("GPU", NB, 8, 24, B)
+    lay = R.plain_layout(NB, L, Hkv, B, D)
+    arena = np.zeros(2 * NB * lay.block_elems, dtype=np.float16)
+    ct, st_ = RO.rotary_tables(D, 1024)
+    builder = StepStateBuilder(8, 1024, Hkv, D, torch.from_numpy(ct).to(cuda), torch.from_numpy(st_).to(cuda))
+    model, engine = Cfg(num_layers=L, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=D), Cfg(block_size=B, max_blocks_per_seq=24)
+    rng = np.random.default_rng(11)
+    arrivals = {0: [(3, 37), (5, 120)], 1: [(0, 16)], 3: [(6, 75), (1, 1)], 5: [(2, 200)]}      # step -> (seq id, prompt)
+    finish = {4: [5], 6: [3, 0]}
+    lens = {}
+    for step in range(8):
+        for sid in finish.get(step, []):
+            ids_t = torch.tensor([sid], dtype=torch.int32, device=cuda)
+            bm.free_blocks_for_seqs(ids_t)
+            ob.free_blocks_for_seqs(np.asarray([sid]))
+            del lens[sid]
+        new = arrivals.get(step, [])
+        running = sorted(lens)
+        p_lens = [n for _, n in new]
+        d_lens = [lens[s] + 1 for s in running]
+        ids = [s for s, _ in new] + running
+        state = builder.build(p_lens, ids, d_lens, block_manager=bm)
+        ob.allocate_blocks_for_seqs(np.asarray(ids), np.asarray(p_lens + d_lens))
+        assert_state_equal(manager_state(bm), ob.snapshot(), f"step {step}: allocation")
+        P, n = sum(p_lens), len(d_lens)
+        T = P + n
+        pos = _positions(p_lens, d_lens)
+        cos, sin = np.ascontiguousarray(ct[pos]), np.ascontiguousarray(st_[pos])
+        starts = np.cumsum(p_lens) - np.asarray(p_lens) if p_lens else np.zeros(0, dtype=np.int64)
+        for layer in range(L):
+            q, k, v = rand_f16(rng, T, Hq, D), rand_f16(rng, T, Hkv, D), rand_f16(rng, T, Hkv, D)
+            qg, kg, vg = (torch.from_numpy(x).to(cuda) for x in (q, k, v))
+            o = torch.full((T, Hq * D), float("nan"), dtype=torch.float16, device=cuda)
+            attention_section(qg, kg, vg, o, pool.k_cache, pool.v_cache, pool.k_cache_new, pool.v_cache_new,
+                              bm.block_table, model, engine, state, layer)
+            RO.rotary_embedding_inplace(q, k, cos, sin)
+            R.store_kvcache(arena, lay, k, v, ob.block_table, np.asarray(ids), len(p_lens), P, starts,
+                            np.asarray(p_lens), np.asarray(d_lens), layer)
+            got = o.cpu().numpy().reshape(T, Hq, D)
+            if P:
+                want = R.prefill_attention(q[:P], k[:P], v[:P], starts, np.asarray(p_lens), D ** -0.5, math="np32")
+                assert_attn_close(got[:P], np.asarray(want), f"step {step} layer {layer}: prefill rows")
+            if n:
+                want = R.paged_attention(q[P:], arena, lay, ob.block_table, np.asarray(running), np.asarray(d_lens),
+                                         D ** -0.5, layer)
+                assert_attn_close(got[P:], np.asarray(want), f"step {step} layer {layer}: decode rows")
+        half = NB * lay.block_elems
+        assert np.array_equal(bits(pool.k_cache).reshape(-1), arena[:half].view(np.uint16)), f"step {step}: K pool"
+        assert np.array_equal(bits(pool.v_cache).reshape(-1), arena[half:].view(np.uint16)), f"step {step}: V pool"
+        for sid, n_tok in new:
+            lens[sid] = n_tok
+        for sid in running:
+            lens[sid] += 1
