@@ -182,7 +182,7 @@ def bench_decode(args):
     else:                                         # as ElasticKVPool creates them: two zeroed allocations, the V base
         from morphserve_amd.kv_placement import allocate_kv_caches   # a few KiB in where the gather measures faster
         k_cache, v_cache, kv_placement = allocate_kv_caches(num_blocks, shape[1:], dev, zero_init=True,
-                                                            tune=not args.no_placement_tuning)
+                                                            tune=False if args.no_placement_tuning else None)
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     live_t = torch.from_numpy(live).to(dev)

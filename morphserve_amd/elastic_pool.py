@@ -30,7 +30,7 @@ class ElasticKVPool:
 
     def __init__(self, num_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int,
-                 device: str = "cuda", zero_init: bool = True, tune_placement: bool = True):
+                 device: str = "cuda", zero_init: bool = True, tune_placement: Optional[bool] = None):
         _capi.lib()
         self.device = torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)

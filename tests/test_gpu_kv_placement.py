@@ -62,9 +62,12 @@ def test_kernels_on_an_offset_v_pool(cuda, offset_bytes):
 
 
 def test_elastic_pool_records_its_placement(cuda):
-    pool = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda")
+    pool = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda",
+                         tune_placement=True)
     assert pool.kv_placement["tuned"] and pool.v_cache.is_contiguous()
     assert pool.descriptor().v_base == pool.v_cache.data_ptr()
     plain = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda",
                           tune_placement=False)
     assert plain.kv_placement == {"v_offset_bytes": 0, "tuned": False} and plain.v_cache.storage_offset() == 0
+    small = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda")
+    assert small.kv_placement == {"v_offset_bytes": 0, "tuned": False}      # 128 MiB per tensor: left alone by default
