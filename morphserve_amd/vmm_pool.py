@@ -106,6 +106,7 @@ class VmmKVPool(ElasticKVPool):
         self._v_arena = _Arena(max_blocks * self.block_bytes, chunk_blocks * self.block_bytes)
         self.k_cache_new, self.v_cache_new = [], []          # never used: the pool is one tensor
         self.kv_cache_new_block_size = 0
+        self.kv_placement = {"v_offset_bytes": 0, "tuned": False}     # two reservations: nothing to choose
         self.block_manager = BlockManager("GPU", num_blocks, max_seqs_in_block_table, max_blocks_per_seq,
                                           block_size, device=device)
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
