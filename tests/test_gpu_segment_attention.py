@@ -214,3 +214,40 @@ def test_attention_through_the_strided_convention(cuda, Hq, Hkv, variant, tps):
         lib.mkv_set_decode_variant(0)
     assert np.array_equal(bits(c.g), bits(c.arena)), "whole arena after the fused append (strided pool)"
     assert_attn_close(o.cpu().numpy(), c.oracle(q), f"fused append, strided pool, {splits} splits")
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (32, 8)])
+def test_attention_section_mixed_batch_over_segments(cuda, Hq, Hkv):
+    """The layer's whole attention section (rotary + append of every row, prefill attention, decode attention)
+    on a mixed batch whose blocks lie in the base pool and in all three segments."""
+    from morphserve_amd import attention_section
+    c = SegCase(cuda, 120 + Hq, Hq, Hkv)
+    rng = np.random.default_rng(Hq + 5)
+    pre, dec = [2, 3], [0, 1, 4, 5, 6]                     # the 16- and 17-token sequences arrive as prompts
+    p_lens = c.lens[pre].tolist()
+    d_lens = c.lens[dec].tolist()
+    ids = c.seq_ids[pre + dec]
+    P, n = sum(p_lens), len(dec)
+    T = P + n
+    q, k, v = rand_f16(rng, T, Hq, 128), rand_f16(rng, T, Hkv, 128), rand_f16(rng, T, Hkv, 128)
+    ct, st_ = RO.rotary_tables(128, 2048)
+    pos = np.concatenate([np.arange(x) for x in p_lens] + [np.asarray(d_lens) - 1])
+    cos, sin = np.ascontiguousarray(ct[pos]), np.ascontiguousarray(st_[pos])
+    state = c.state(p_lens, d_lens, ids.tolist())
+    state.position_cos = torch.from_numpy(cos).to(cuda)
+    state.position_sin = torch.from_numpy(sin).to(cuda)
+    qg, kg, vg = (torch.from_numpy(x).to(cuda) for x in (q, k, v))
+    o = torch.full((T, Hq * 128), float("nan"), dtype=torch.float16, device=cuda)
+    attention_section(qg, kg, vg, o, c.kc, c.vc, c.k_new, c.v_new, c.bt, c.model, c.engine, state, LAYER)
+    torch.cuda.synchronize()
+    RO.rotary_embedding_inplace(q, k, cos, sin)
+    starts = np.cumsum(p_lens) - np.asarray(p_lens)
+    R.store_kvcache(c.arena, c.lay, k, v, c.table, ids, len(pre), P, starts, np.asarray(p_lens), np.asarray(d_lens),
+                    LAYER)
+    assert np.array_equal(bits(c.g), bits(c.arena)), "whole arena after rotary + append of the mixed batch"
+    assert np.array_equal(bits(qg), bits(q)) and np.array_equal(bits(kg), bits(k))
+    got = o.cpu().numpy().reshape(T, Hq, 128)
+    want_p = R.prefill_attention(q[:P], k[:P], v[:P], starts, np.asarray(p_lens), 128 ** -0.5, math="np32")
+    assert_attn_close(got[:P], np.asarray(want_p), "prefill rows")
+    want_d = R.paged_attention(q[P:], c.arena, c.lay, c.table, ids[len(pre):], np.asarray(d_lens), 128 ** -0.5, LAYER)
+    assert_attn_close(got[P:], np.asarray(want_d), "decode rows over segments")
