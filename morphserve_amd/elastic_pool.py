@@ -73,8 +73,11 @@ class ElasticKVPool:
         lib = _capi.lib()
         stream = _capi.current_stream()
         if k_seg is None:
-            k_seg = torch.empty((seg_blocks, *self.shape_tail), dtype=torch.float16, device=self.device)
-            v_seg = torch.empty((seg_blocks, *self.shape_tail), dtype=torch.float16, device=self.device)
+            shape = (seg_blocks, *self.shape_tail)
+            k_seg = torch.empty(shape, dtype=torch.float16, device=self.device)
+            off = self.kv_placement["v_offset_bytes"] // 2       # the base pool's K-to-V stagger serves its segments too
+            numel = k_seg.numel()
+            v_seg = torch.empty(numel + off, dtype=torch.float16, device=self.device)[off:].view(shape)
         assert tuple(k_seg.shape) == (seg_blocks, *self.shape_tail) and k_seg.is_contiguous()
         assert tuple(v_seg.shape) == (seg_blocks, *self.shape_tail) and v_seg.is_contiguous()
         nbytes = seg_blocks * self.block_bytes
