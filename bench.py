@@ -87,6 +87,9 @@ def parse_args():
                          "batch of chunks over PREFIX tokens already in a paged cache")
     ap.add_argument("--no-placement-tuning", action="store_true",
                     help="decode workloads, diagnostic: the V pool starts at its allocation's base (no probing of offsets)")
+    ap.add_argument("--settle-seconds", type=float, default=None,
+                    help="decode workloads: how long pool creation waits before its one retry when the placement probe "
+                         "reads a recently recycled allocation (default: the library's 12 s; 0 = never retry)")
     ap.add_argument("--prefill-kv-heads", type=int, default=32,
                     help="prefill_shapes workload, whole prompts: kv heads behind the 32 q heads (1 = every q head reads the "
                          "same K/V, which then always comes out of the L2s: the same matrix work without the K/V traffic)")
@@ -182,7 +185,8 @@ def bench_decode(args):
     else:                                         # as ElasticKVPool creates them: two zeroed allocations, the V base
         from morphserve_amd.kv_placement import allocate_kv_caches   # a few KiB in where the gather measures faster
         k_cache, v_cache, kv_placement = allocate_kv_caches(num_blocks, shape[1:], dev, zero_init=True,
-                                                            tune=False if args.no_placement_tuning else None)
+                                                            tune=False if args.no_placement_tuning else None,
+                                                            settle_seconds=args.settle_seconds)
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     live_t = torch.from_numpy(live).to(dev)
@@ -509,7 +513,8 @@ def bench_resize(args):
     ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1          # 32k -> 96k -> 40k blocks of 2 MiB
     rng = np.random.default_rng(args.seed)
     _warm_resize_kernels(dev, L, HKV, B, D)
-    pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256)
+    pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256,
+                         tune_placement=False if args.no_placement_tuning else None, settle_seconds=args.settle_seconds)
     blk_bytes = pool.block_bytes
     _capi.prof_reset()
     _capi.prof_enable(True)
@@ -569,7 +574,7 @@ def bench_resize(args):
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"cfg3_resize: 2 MiB blocks (32 layers x 8 kv heads x 16 x 128 fp16, K+V), "
                                f"grow {ORG}->{total} (zero fill), {len(live)} live scattered, shrink to {new_n}"},
-        "moves": moves, "moved_GiB": round(moved_bytes / 2 ** 30, 2),
+        "moves": moves, "moved_GiB": round(moved_bytes / 2 ** 30, 2), "kv_placement": pool.kv_placement,
         "expand_s": round(expand_s, 4), "zero_fill_GBs": round(fill_gbs, 1),
         "pct_of_hbm_peak": round(100 * whole / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel", "achieved": round(achieved, 1),
@@ -1674,6 +1679,7 @@ def main():
         out["resize"] = {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"],
                          "unit": r["unit"], "ms": r["ms_per_step"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
                          "moves": r["moves"], "moved_GiB": r["moved_GiB"], "expand_s": r["expand_s"],
+                         "kv_placement": r["kv_placement"],
                          "zero_fill_GBs": r["zero_fill_GBs"], "dtype": r["dtype"], "roofline": r["roofline"],
                          **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})}
     print(json.dumps(out))

@@ -30,14 +30,16 @@ class ElasticKVPool:
 
     def __init__(self, num_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int,
-                 device: str = "cuda", zero_init: bool = True, tune_placement: Optional[bool] = None):
+                 device: str = "cuda", zero_init: bool = True, tune_placement: Optional[bool] = None,
+                 settle_seconds: Optional[float] = None):
         _capi.lib()
         self.device = torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
         # K and V as the reference creates them (model.py:187-190); the V base may sit a few KiB into its
         # allocation where the decode gather measures faster that way (kv_placement)
         self.k_cache, self.v_cache, self.kv_placement = allocate_kv_caches(
-            num_blocks, self.shape_tail, device, zero_init=zero_init, tune=tune_placement)
+            num_blocks, self.shape_tail, device, zero_init=zero_init, tune=tune_placement,
+            settle_seconds=settle_seconds)
         self.k_cache_new: List[torch.Tensor] = []
         self.v_cache_new: List[torch.Tensor] = []
         self.kv_cache_new_block_size = 0

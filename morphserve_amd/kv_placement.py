@@ -17,6 +17,7 @@ effect was measured on 64-186 GiB pools; on a pool of a few hundred MiB the prob
 from __future__ import annotations
 
 import ctypes as C
+import time
 from typing import Dict, Optional, Sequence, Tuple
 
 import torch
@@ -28,6 +29,8 @@ CANDIDATE_OFFSETS = (0, 4096, 8192, 12288, 20480)
 SLACK_BYTES = 32768
 MIN_BLOCKS_TO_TUNE = 4096
 MIN_BYTES_TO_TUNE = 16 << 30
+SETTLE_SECONDS = 12.0
+SETTLE_BELOW_GBS = 6080.0           # probe on a 128 GiB pool: 6140-6190 GB/s on settled memory, 5650-6035 on recycled memory
 
 
 def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Sequence[int]) -> float:
@@ -54,19 +57,46 @@ def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Seque
 
 
 def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], device, zero_init: bool = True,
-                       tune: Optional[bool] = None, seed: int = 0) -> Tuple[torch.Tensor, torch.Tensor, Dict]:
-    """``(k_cache, v_cache, info)`` with ``k_cache, v_cache : [num_blocks, L, Hkv, B, D]`` fp16."""
+                       tune: Optional[bool] = None, seed: int = 0,
+                       settle_seconds: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor, Dict]:
+    """``(k_cache, v_cache, info)`` with ``k_cache, v_cache : [num_blocks, L, Hkv, B, D]`` fp16.
+
+    ``settle_seconds`` (``None``: ``SETTLE_SECONDS`` whenever the probe runs, 0: never): for some seconds after
+    a large amount of device memory has been freed -- by this process or by one that has just exited -- the
+    driver hands out memory on which the gather runs 2-7 % slower for as long as the allocation lives; an
+    allocation made ten seconds later is as fast as the first one of a freshly started machine.  When the probe
+    reads less than ``SETTLE_BELOW_GBS`` the pool is therefore given back, the call sleeps ``settle_seconds`` and
+    allocates and probes once more (never more than once; the second allocation is kept whatever it reads)."""
     L, hkv, bsz, d = shape_tail
     device = torch.device(device)
+    shape = (num_blocks, L, hkv, bsz, d)
+    numel = num_blocks * L * hkv * bsz * d
+    supported = bsz == 16 and d == 128 and device.type == "cuda"
+    if tune is None:
+        tune = numel * 2 >= MIN_BYTES_TO_TUNE
+    tune = bool(tune and supported and num_blocks >= MIN_BLOCKS_TO_TUNE)
+    if settle_seconds is None:
+        settle_seconds = SETTLE_SECONDS
+    k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
+    if tune and settle_seconds > 0 and info["probe_GBs"] < SETTLE_BELOW_GBS:
+        first = info["probe_GBs"]
+        del k_cache, v_cache
+        torch.cuda.synchronize(device)
+        torch.cuda.empty_cache()
+        time.sleep(settle_seconds)
+        k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
+        info["settled"] = {"first_probe_GBs": first, "waited_s": settle_seconds}
+    return k_cache, v_cache, info
+
+
+def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tune: bool, seed: int):
+    L, hkv, bsz, d = shape_tail
     alloc = torch.zeros if zero_init else torch.empty
     shape = (num_blocks, L, hkv, bsz, d)
     numel = num_blocks * L * hkv * bsz * d
     k_cache = alloc(shape, dtype=torch.float16, device=device)
     info: Dict = {"v_offset_bytes": 0, "tuned": False}
-    supported = bsz == 16 and d == 128 and device.type == "cuda"
-    if tune is None:
-        tune = numel * 2 >= MIN_BYTES_TO_TUNE
-    if not (tune and supported and num_blocks >= MIN_BLOCKS_TO_TUNE):
+    if not tune:
         return k_cache, alloc(shape, dtype=torch.float16, device=device), info
     v_flat = alloc(numel + SLACK_BYTES // 2, dtype=torch.float16, device=device)
     # the probe: as many sequences as put two workgroups on every CU, 64 blocks each, block ids drawn over
@@ -91,5 +121,8 @@ def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], d
     best = min(timings, key=timings.get)
     if timings[best] > 0.995 * timings[0]:          # within the noise of the probe: keep the plain placement
         best = 0
-    info = {"v_offset_bytes": best, "tuned": True, "probe_us_per_launch": {str(k): round(v, 2) for k, v in timings.items()}}
+    probe_bytes = n * per_seq * hkv * 2 * bsz * d * 2                 # every K and V slab of the probe batch once
+    info = {"v_offset_bytes": best, "tuned": True,
+            "probe_us_per_launch": {str(k): round(v, 2) for k, v in timings.items()},
+            "probe_GBs": round(probe_bytes / timings[best] / 1e3, 1)}
     return k_cache, v_flat[best // 2: best // 2 + numel].view(shape), info
