@@ -30,7 +30,11 @@ SLACK_BYTES = 32768
 MIN_BLOCKS_TO_TUNE = 4096
 MIN_BYTES_TO_TUNE = 16 << 30
 SETTLE_SECONDS = 12.0
-SETTLE_BELOW_GBS = 6080.0           # probe on a 128 GiB pool: 6140-6190 GB/s on settled memory, 5650-6035 on recycled memory
+# The probe on settled / recycled memory, K + V pools of 128 GiB: 6140-6190 / 5650-6035 GB/s; of 64 GiB: 6320-6370 /
+# 6000-6090 GB/s (a smaller pool gathers faster).  The line between them, per GiB of pool, clamped:
+SETTLE_BELOW_GBS = 6080.0
+SETTLE_BELOW_GBS_PER_GIB = -1.9     # relative to a 128 GiB pool
+SETTLE_BELOW_RANGE = (5900.0, 6250.0)
 
 
 def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Sequence[int]) -> float:
@@ -65,7 +69,8 @@ def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], d
     a large amount of device memory has been freed -- by this process or by one that has just exited -- the
     driver hands out memory on which the gather runs 2-7 % slower for as long as the allocation lives; an
     allocation made ten seconds later is as fast as the first one of a freshly started machine.  When the probe
-    reads less than ``SETTLE_BELOW_GBS`` the pool is therefore given back, the call sleeps ``settle_seconds`` and
+    reads less than a threshold calibrated on this GPU (``SETTLE_BELOW_GBS`` for a 128 GiB pool, a little more for a
+    smaller one) the pool is therefore given back, the call sleeps ``settle_seconds`` and
     allocates and probes once more (never more than once; the second allocation is kept whatever it reads)."""
     L, hkv, bsz, d = shape_tail
     device = torch.device(device)
@@ -78,7 +83,7 @@ def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], d
     if settle_seconds is None:
         settle_seconds = SETTLE_SECONDS
     k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
-    if tune and settle_seconds > 0 and info["probe_GBs"] < SETTLE_BELOW_GBS:
+    if tune and settle_seconds > 0 and info["probe_GBs"] < _settle_threshold(2 * numel * 2):
         first = info["probe_GBs"]
         del k_cache, v_cache
         torch.cuda.synchronize(device)
@@ -87,6 +92,13 @@ def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], d
         k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
         info["settled"] = {"first_probe_GBs": first, "waited_s": settle_seconds}
     return k_cache, v_cache, info
+
+
+def _settle_threshold(pool_bytes: int) -> float:
+    if SETTLE_BELOW_GBS <= 0 or SETTLE_BELOW_GBS >= 1e9:          # switched off / forced (tests)
+        return SETTLE_BELOW_GBS
+    thr = SETTLE_BELOW_GBS + SETTLE_BELOW_GBS_PER_GIB * (pool_bytes / 2 ** 30 - 128.0)
+    return min(max(thr, SETTLE_BELOW_RANGE[0]), SETTLE_BELOW_RANGE[1])
 
 
 def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tune: bool, seed: int):
