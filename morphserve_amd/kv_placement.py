@@ -30,11 +30,11 @@ SLACK_BYTES = 32768
 MIN_BLOCKS_TO_TUNE = 4096
 MIN_BYTES_TO_TUNE = 16 << 30
 SETTLE_SECONDS = 12.0
-# The probe on settled / recycled memory, K + V pools of 128 GiB: 6140-6190 / 5650-6035 GB/s; of 64 GiB: 6320-6370 /
-# 6000-6090 GB/s (a smaller pool gathers faster).  The line between them, per GiB of pool, clamped:
-SETTLE_BELOW_GBS = 6080.0
-SETTLE_BELOW_GBS_PER_GIB = -1.9     # relative to a 128 GiB pool
-SETTLE_BELOW_RANGE = (5900.0, 6250.0)
+# The probe on settled / recycled memory, K + V pools of 128 GiB: 6140-6190 / 5650-6035 GB/s; of 186 GiB: 6180-6200 /
+# 5930; of 64 GiB: 6320-6370 / 6000-6090 GB/s (a smaller pool gathers faster).  The line between them:
+SETTLE_BELOW_GBS = 6080.0           # pools of 128 GiB and more
+SETTLE_BELOW_GBS_PER_GIB = -1.9     # added per GiB under 128
+SETTLE_BELOW_MAX = 6250.0
 
 
 def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Sequence[int]) -> float:
@@ -97,8 +97,8 @@ def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], d
 def _settle_threshold(pool_bytes: int) -> float:
     if SETTLE_BELOW_GBS <= 0 or SETTLE_BELOW_GBS >= 1e9:          # switched off / forced (tests)
         return SETTLE_BELOW_GBS
-    thr = SETTLE_BELOW_GBS + SETTLE_BELOW_GBS_PER_GIB * (pool_bytes / 2 ** 30 - 128.0)
-    return min(max(thr, SETTLE_BELOW_RANGE[0]), SETTLE_BELOW_RANGE[1])
+    thr = SETTLE_BELOW_GBS + SETTLE_BELOW_GBS_PER_GIB * min(0.0, pool_bytes / 2 ** 30 - 128.0)
+    return min(thr, SETTLE_BELOW_MAX)
 
 
 def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tune: bool, seed: int):
