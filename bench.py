@@ -59,7 +59,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
                              "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover", "step_state"])
+                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover", "step_state", "slab_gather"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -1469,6 +1469,62 @@ def bench_copy_calibration(args):
 
 
 # ---------------------------------------------------------------------------------
+def bench_slab_gather(args):
+    """What the memory system gives the decode gather: random 4 KiB slab reads and nothing else (2 GiB per launch),
+    against the bytes in flight per CU, the footprint (one 64 GiB allocation or two) and which XCDs read which
+    allocation (``mkv_diag_slab_gather``)."""
+    import torch
+    from morphserve_amd import _capi
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib, stream = _capi.lib(), _capi.current_stream()
+    gib = 1 << 30
+    bufs = [torch.ones(64 * gib, dtype=torch.uint8, device=dev) for _ in range(2)]
+    spacer = torch.empty(32 * gib, dtype=torch.uint8, device=dev)
+    bufs.append(torch.ones(64 * gib, dtype=torch.uint8, device=dev))      # 96 GiB below the first one
+    del spacer
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    slabs = 64 * gib // 4096
+    per, total = 64, 1 << 19                                               # 2 GiB per launch
+
+    def rate(a, b, loads, wpc, by_xcd=0, mask=0):
+        def launch():
+            _capi.check(lib.mkv_diag_slab_gather(a.data_ptr(), b.data_ptr(), slabs, total // per, per, loads, wpc, by_xcd,
+                                                 mask, sink.data_ptr(), stream))
+        launch()
+        launch()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            launch()
+        e1.record()
+        e1.synchronize()
+        return round(total * 4096 * args.steps / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
+
+    in_flight = {}
+    for tag, b in (("one allocation (64 GiB)", bufs[0]), ("two allocations (128 GiB)", bufs[1])):
+        in_flight[tag] = {f"{wpc} workgroups per CU x {loads} loads per thread = {wpc * 256 * loads * 16 // 1024} KiB per CU":
+                          rate(bufs[0], b, loads, wpc) for wpc in (1, 2, 4, 8) for loads in (1, 2, 4, 8)}
+    by_xcd = {}
+    for tag, b in (("second allocation = the neighbour", bufs[1]), ("second allocation = 96 GiB further down", bufs[2])):
+        by_xcd[tag] = {name: rate(bufs[0], b, 4, 8, 1, mask) for name, mask in
+                       (("all XCDs read the first", 0x00), ("all XCDs read the second", 0xFF),
+                        ("XCDs 0-3 the first, 4-7 the second", 0xF0), ("XCDs 0-3 the second, 4-7 the first", 0x0F),
+                        ("even XCDs the first, odd the second", 0xAA), ("XCDs 0,1,4,5 the first, 2,3,6,7 the second", 0xCC))}
+    best = max(in_flight["two allocations (128 GiB)"].values())
+    return {
+        "metric": "random 4 KiB slab reads, nothing else in the kernel, GB/s, 1 MI355X",
+        "value": best, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 2,
+        "ms_per_step": round(total * 4096 / best / 1e6, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "slab_gather: 2 GiB of random 4 KiB slabs per launch out of 64 GiB allocations"},
+        "GBs_by_bytes_in_flight": in_flight, "GBs_by_xcd_group": by_xcd,
+        "roofline": {"bound": "hbm", "kernel": "diag_slab_gather_kernel<U>", "achieved": best, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(best / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+
+
 def bench_step_state(args):
     """Host time of a step's preparation (MorphServe/worker/model.py:318-436): the reference's way -- one device
     tensor per host list, an arange per prefill sequence, two gathers -- against ``StepStateBuilder`` (one pinned
@@ -1667,7 +1723,7 @@ def main():
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
              "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
              "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving,
-             "timeline": bench_timeline, "layer_handover": bench_layer_handover, "step_state": bench_step_state}
+             "timeline": bench_timeline, "layer_handover": bench_layer_handover, "step_state": bench_step_state, "slab_gather": bench_slab_gather}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
         # the second target of the path in the same process and the same JSON line: the decode pool is gone

@@ -51,6 +51,16 @@ int mkv_set_prefill_variant(int32_t waves);
 int mkv_diag_mfma_loop(int32_t mode, int32_t iters, const void* data, void* sink, double* flops,
                        void* stream);
 
+/* What the memory system gives a gather of 4 KiB slabs (no counterpart in the reference): `workgroups`
+ * workgroups of 256 threads read slabs_per_wg slabs each, loads_in_flight (1, 2, 4, 8) per thread at a
+ * time, workgroups_per_cu (1 ... 8) resident per CU; the slab is a hash of (workgroup, i) over
+ * slabs_in_buf (a power of two) slabs of buffer a or b (4 KiB aligned, slabs_in_buf * 4096 bytes each).
+ * by_xcd = 0: the buffer is one bit of the hash; by_xcd != 0: workgroups on XCD x (= workgroup id mod 8)
+ * read b when bit x of xcd_mask is set, else a.  sink: 4 bytes of device scratch.  Reads only. */
+int mkv_diag_slab_gather(const void* a, const void* b, uint64_t slabs_in_buf, int32_t workgroups,
+                         int32_t slabs_per_wg, int32_t loads_in_flight, int32_t workgroups_per_cu, int32_t by_xcd,
+                         uint32_t xcd_mask, void* sink, void* stream);
+
 /* Per-workgroup time stamps of the attention kernels.  buf: device memory of
  * max_workgroups * MKV_TIMELINE_POINTS int64, zeroed by the caller; NULL switches
  * the stamps off.  While set, every launch of the prefill kernel and of the decode

@@ -87,6 +87,7 @@ PROTOTYPES = {
     "mkv_swap_blocks_device_ids": [_P, _P, _I64, _I32, _PP, _P, _P, _I64, _P],
     "mkv_diag_mfma_loop": [_I32, _I32, _P, _P, C.POINTER(C.c_double), _P],
     "mkv_diag_timeline": [_P, _I64],
+    "mkv_diag_slab_gather": [_P, _P, _U64, _I32, _I32, _I32, _I32, _I32, C.c_uint32, _P, _P],
     "mkv_prof_enable": [_I32],
     "mkv_prof_reset": [],
     "mkv_prof_collect": [_I32, C.POINTER(_I64), C.POINTER(C.c_double)],

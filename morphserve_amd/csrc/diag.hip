@@ -88,9 +88,71 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     sink[blockIdx.x * blockDim.x + tid] = keep;
 }
 
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+// Random 4 KiB slab reads and nothing else: what the memory system gives the decode gather.  Workgroup w reads
+// slabs_per_wg slabs, U at a time; the slab comes from a multiplicative hash of (w, i), its buffer from one hash bit
+// or, with by_xcd, from bit (w % 8) of xcd_mask (the XCD a workgroup of a 1-D grid runs on).
+template <int U>
+__global__ __launch_bounds__(256) void diag_slab_gather_kernel(const char* __restrict__ a, const char* __restrict__ b,
+                                                               uint64_t slabs_in_buf, int32_t slabs_per_wg,
+                                                               int32_t by_xcd, uint32_t xcd_mask,
+                                                               uint32_t* __restrict__ sink) {
+    extern __shared__ char occupancy_pad[];                 // sized by the launcher to limit the workgroups per CU
+    const uint32_t w = blockIdx.x;
+    v4u acc = (v4u){0u, 0u, 0u, 0u};
+    for (int i = 0; i < slabs_per_wg; i += U) {
+        v4u v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t h = ((uint64_t)w * (uint64_t)slabs_per_wg + (uint64_t)(i + u)) * 0x9E3779B97F4A7C15ull;
+            const uint64_t slab = (h >> 20) & (slabs_in_buf - 1);
+            const bool second = by_xcd ? ((xcd_mask >> (w & 7u)) & 1u) != 0 : ((h >> 50) & 1u) != 0;
+            v[u] = __builtin_nontemporal_load((const v4u*)((second ? b : a) + slab * 4096) + threadIdx.x);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u];
+        asm volatile("" : "+v"(acc.x));                     // the next group's loads wait for this one
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345677u) {   // keeps the loads; practically never true
+        sink[0] = 1;
+        occupancy_pad[0] = 1;
+    }
+}
+
 }  // namespace mkv
 
 extern "C" {
+
+int mkv_diag_slab_gather(const void* a, const void* b, uint64_t slabs_in_buf, int32_t workgroups,
+                         int32_t slabs_per_wg, int32_t loads_in_flight, int32_t workgroups_per_cu, int32_t by_xcd,
+                         uint32_t xcd_mask, void* sink, void* stream) {
+    MKV_REQUIRE(a && b && sink, "NULL argument");
+    MKV_REQUIRE(slabs_in_buf > 0 && (slabs_in_buf & (slabs_in_buf - 1)) == 0, "slabs_in_buf must be a power of two");
+    MKV_REQUIRE(workgroups > 0 && slabs_per_wg > 0, "bad grid");
+    MKV_REQUIRE(loads_in_flight == 1 || loads_in_flight == 2 || loads_in_flight == 4 || loads_in_flight == 8,
+                "loads_in_flight must be 1, 2, 4 or 8");
+    MKV_REQUIRE(slabs_per_wg % loads_in_flight == 0, "slabs_per_wg must be a multiple of loads_in_flight");
+    MKV_REQUIRE(workgroups_per_cu >= 1 && workgroups_per_cu <= 8, "workgroups_per_cu must be 1 ... 8");
+    MKV_REQUIRE((((uintptr_t)a | (uintptr_t)b) & 4095) == 0, "buffers must be 4 KiB aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const int lds = 160 * 1024 / workgroups_per_cu - 1024;  // that many workgroups fit the CU's 160 KiB
+    const dim3 grid((unsigned)workgroups), block(256);
+#define MKV_SLAB_GATHER(U)                                                                                          \
+    do {                                                                                                            \
+        MKV_HIP(hipFuncSetAttribute((const void*)mkv::diag_slab_gather_kernel<U>,                                    \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));                               \
+        hipLaunchKernelGGL(mkv::diag_slab_gather_kernel<U>, grid, block, lds, s, (const char*)a, (const char*)b,     \
+                           slabs_in_buf, slabs_per_wg, by_xcd, xcd_mask, (uint32_t*)sink);                           \
+    } while (0)
+    if (loads_in_flight == 1) MKV_SLAB_GATHER(1);
+    if (loads_in_flight == 2) MKV_SLAB_GATHER(2);
+    if (loads_in_flight == 4) MKV_SLAB_GATHER(4);
+    if (loads_in_flight == 8) MKV_SLAB_GATHER(8);
+#undef MKV_SLAB_GATHER
+    MKV_HIP(hipGetLastError());
+    return MKV_OK;
+}
 
 int mkv_diag_mfma_loop(int32_t mode, int32_t iters, const void* data, void* sink, double* flops,
                        void* stream) {
