@@ -179,9 +179,9 @@ def bench_decode(args):
     if args.pool_backing == "vmm":                # one tensor over HIP virtual memory
         from morphserve_amd import VmmKVPool
         vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq,
-                             chunk_blocks=args.vmm_chunk_blocks)
+                             chunk_blocks=args.vmm_chunk_blocks, settle_seconds=args.settle_seconds)
         k_cache, v_cache = vmm_pool.k_cache, vmm_pool.v_cache
-        kv_placement = {"v_offset_bytes": 0, "tuned": False}
+        kv_placement = vmm_pool.kv_placement
     else:                                         # as ElasticKVPool creates them: two zeroed allocations, the V base
         from morphserve_amd.kv_placement import allocate_kv_caches   # a few KiB in where the gather measures faster
         k_cache, v_cache, kv_placement = allocate_kv_caches(num_blocks, shape[1:], dev, zero_init=True,

@@ -101,6 +101,39 @@ def _settle_threshold(pool_bytes: int) -> float:
     return min(thr, SETTLE_BELOW_MAX)
 
 
+def _make_probe(num_blocks: int, shape_tail, device, seed: int):
+    """The probe batch: as many sequences as put two workgroups on every CU, 64 blocks each, block ids drawn over
+    the whole pool; one q head per kv head (the vector-ALU kernel reads memory exactly as the matrix one does)."""
+    L, hkv, bsz, d = shape_tail
+    n = max(1, 512 // hkv)
+    per_seq = min(64, num_blocks // n)
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed)
+    bt = torch.randperm(num_blocks, generator=gen)[:n * per_seq].to(torch.int32).view(n, per_seq).to(device)
+    ids = torch.arange(n, dtype=torch.int32, device=device)
+    lens_t = torch.full((n,), per_seq * 16, dtype=torch.int32, device=device)
+    q = torch.zeros((n, hkv, d), dtype=torch.float16, device=device)
+    o = torch.empty((n, hkv, d), dtype=torch.float16, device=device)
+    layers = list(range(0, L, max(1, L // 4)))[:4]
+    probe_bytes = n * per_seq * hkv * 2 * bsz * d * 2                 # every K and V slab of the probe batch once
+    return (bt, ids, lens_t, q, o, n, hkv), layers, probe_bytes
+
+
+def probe_gather_GBs(k_cache: torch.Tensor, v_cache: torch.Tensor, seed: int = 0) -> float:
+    """GB/s of the probe gather over an existing pool (best of three passes): the figure ``allocate_kv_caches``
+    compares with its threshold, for pools whose memory is obtained in another way."""
+    num_blocks = int(k_cache.shape[0])
+    shape_tail = tuple(int(x) for x in k_cache.shape[1:])
+    probe, layers, probe_bytes = _make_probe(num_blocks, shape_tail, k_cache.device, seed)
+    best = min(_probe_us(k_cache, v_cache, probe, layers) for _ in range(3))
+    return round(probe_bytes / best / 1e3, 1)
+
+
+def settle_threshold_GBs(pool_bytes: int) -> float:
+    """Below this probe rate a pool of ``pool_bytes`` (K and V together) is taken to lie on recycled memory."""
+    return _settle_threshold(pool_bytes)
+
+
 def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tune: bool, seed: int):
     L, hkv, bsz, d = shape_tail
     alloc = torch.zeros if zero_init else torch.empty
@@ -111,20 +144,7 @@ def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tu
     if not tune:
         return k_cache, alloc(shape, dtype=torch.float16, device=device), info
     v_flat = alloc(numel + SLACK_BYTES // 2, dtype=torch.float16, device=device)
-    # the probe: as many sequences as put two workgroups on every CU, 64 blocks each, block ids drawn over
-    # the whole pool; one q head per kv head (the vector-ALU kernel reads memory exactly as the matrix one does)
-    n = max(1, 512 // hkv)
-    per_seq = min(64, num_blocks // n)
-    gen = torch.Generator(device="cpu")
-    gen.manual_seed(seed)
-    ids_pool = torch.randperm(num_blocks, generator=gen)[:n * per_seq].to(torch.int32).view(n, per_seq)
-    bt = ids_pool.to(device)
-    ids = torch.arange(n, dtype=torch.int32, device=device)
-    lens_t = torch.full((n,), per_seq * 16, dtype=torch.int32, device=device)
-    q = torch.zeros((n, hkv, d), dtype=torch.float16, device=device)
-    o = torch.empty((n, hkv, d), dtype=torch.float16, device=device)
-    probe = (bt, ids, lens_t, q, o, n, hkv)
-    layers = list(range(0, L, max(1, L // 4)))[:4]
+    probe, layers, probe_bytes = _make_probe(num_blocks, shape_tail, device, seed)
     timings = {off: float("inf") for off in CANDIDATE_OFFSETS}
     for _ in range(3):                              # candidates in turn, three times over: the best of each
         for off in CANDIDATE_OFFSETS:
@@ -133,7 +153,6 @@ def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tu
     best = min(timings, key=timings.get)
     if timings[best] > 0.995 * timings[0]:          # within the noise of the probe: keep the plain placement
         best = 0
-    probe_bytes = n * per_seq * hkv * 2 * bsz * d * 2                 # every K and V slab of the probe batch once
     info = {"v_offset_bytes": best, "tuned": True,
             "probe_us_per_launch": {str(k): round(v, 2) for k, v in timings.items()},
             "probe_GBs": round(probe_bytes / timings[best] / 1e3, 1)}

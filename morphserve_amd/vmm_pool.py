@@ -13,7 +13,8 @@ Same ``BlockManager`` and bookkeeping as ``ElasticKVPool``.
 from __future__ import annotations
 
 import ctypes as C
-from typing import Tuple
+import time
+from typing import Optional, Tuple
 
 import torch
 
@@ -94,7 +95,7 @@ class VmmKVPool(ElasticKVPool):
 
     def __init__(self, num_blocks: int, max_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int, chunk_blocks: int = 64,
-                 device: str = "cuda"):
+                 device: str = "cuda", settle_seconds: Optional[float] = None):
         _capi.lib()
         self.device = torch.device(device, torch.cuda.current_device()) if device == "cuda" else torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
@@ -112,6 +113,34 @@ class VmmKVPool(ElasticKVPool):
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
         self._map(num_blocks)
         self._zero(0, num_blocks)
+        self._settle(num_blocks, settle_seconds)
+
+    def _settle(self, num_blocks: int, settle_seconds: Optional[float]) -> None:
+        """``allocate_kv_caches``' one retry for mapped memory: a large pool whose probe reads recycled memory is
+        unmapped, the call sleeps and maps it again (the K-to-V stagger has no counterpart here: both ranges start
+        on a chunk boundary)."""
+        from . import kv_placement as KP
+        pool_bytes = 2 * num_blocks * self.block_bytes
+        if settle_seconds is None:
+            settle_seconds = KP.SETTLE_SECONDS
+        l, h, b, d = self.shape_tail
+        big = num_blocks * self.block_bytes >= KP.MIN_BYTES_TO_TUNE and num_blocks >= KP.MIN_BLOCKS_TO_TUNE
+        if not (big and b == 16 and d == 128 and settle_seconds > 0):
+            return
+        first = KP.probe_gather_GBs(self.k_cache, self.v_cache)
+        self.kv_placement = {"v_offset_bytes": 0, "tuned": False, "probe_GBs": first}
+        if first >= KP.settle_threshold_GBs(pool_bytes):
+            return
+        torch.cuda.synchronize(self.device)
+        self.k_cache = self.v_cache = None
+        self._k_arena.resize(0)
+        self._v_arena.resize(0)
+        time.sleep(settle_seconds)
+        self._map(num_blocks)
+        self._zero(0, num_blocks)
+        self.kv_placement = {"v_offset_bytes": 0, "tuned": False,
+                             "probe_GBs": KP.probe_gather_GBs(self.k_cache, self.v_cache),
+                             "settled": {"first_probe_GBs": first, "waited_s": settle_seconds}}
 
     # -- mapping ---------------------------------------------------------------------
     def _map(self, num_blocks: int) -> None:
