@@ -95,7 +95,11 @@ class VmmKVPool(ElasticKVPool):
 
     def __init__(self, num_blocks: int, max_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int, chunk_blocks: int = 64,
-                 device: str = "cuda", settle_seconds: Optional[float] = None):
+                 device: str = "cuda", settle_seconds: Optional[float] = None,
+                 v_stagger_bytes: Optional[int] = None):
+        """``v_stagger_bytes``: how far into its range the V tensor starts (a multiple of 4 KiB below the chunk
+        size; it costs one more mapped chunk).  ``None``: chosen by the probe of ``kv_placement`` for pools of
+        ``MIN_BYTES_TO_TUNE`` per tensor and more, 0 otherwise."""
         _capi.lib()
         self.device = torch.device(device, torch.cuda.current_device()) if device == "cuda" else torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
@@ -103,8 +107,18 @@ class VmmKVPool(ElasticKVPool):
         if num_blocks % chunk_blocks or max_blocks % chunk_blocks or not 0 < num_blocks <= max_blocks:
             raise ValueError(f"num_blocks and max_blocks must be multiples of chunk_blocks ({chunk_blocks})")
         self.max_blocks = max_blocks
-        self._k_arena = _Arena(max_blocks * self.block_bytes, chunk_blocks * self.block_bytes)
-        self._v_arena = _Arena(max_blocks * self.block_bytes, chunk_blocks * self.block_bytes)
+        from . import kv_placement as KP
+        chunk = chunk_blocks * self.block_bytes
+        l, h, b, d = self.shape_tail
+        probe_ok = (b == 16 and d == 128 and num_blocks >= KP.MIN_BLOCKS_TO_TUNE
+                    and num_blocks * self.block_bytes >= KP.MIN_BYTES_TO_TUNE)
+        choose = v_stagger_bytes is None and probe_ok and chunk > max(KP.CANDIDATE_OFFSETS)
+        if v_stagger_bytes is not None and (v_stagger_bytes < 0 or v_stagger_bytes % 4096 or v_stagger_bytes >= chunk):
+            raise ValueError("v_stagger_bytes must be a multiple of 4096 below the chunk size")
+        self._v_off = int(v_stagger_bytes or 0)
+        self._v_pad = chunk if (choose or self._v_off) else 0      # the V range is mapped one chunk further
+        self._k_arena = _Arena(max_blocks * self.block_bytes, chunk)
+        self._v_arena = _Arena(max_blocks * self.block_bytes + self._v_pad, chunk)
         self.k_cache_new, self.v_cache_new = [], []          # never used: the pool is one tensor
         self.kv_cache_new_block_size = 0
         self.kv_placement = {"v_offset_bytes": 0, "tuned": False}     # two reservations: nothing to choose
@@ -114,6 +128,30 @@ class VmmKVPool(ElasticKVPool):
         self._map(num_blocks)
         self._zero(0, num_blocks)
         self._settle(num_blocks, settle_seconds)
+        if choose:
+            self._choose_stagger(num_blocks)
+
+    def _choose_stagger(self, num_blocks: int) -> None:
+        """The K-to-V stagger of ``kv_placement``: the V tensor viewed at each candidate offset of its (zeroed) range,
+        the fastest kept unless offset 0 is within the probe's noise of it."""
+        from . import kv_placement as KP
+        probe, layers, probe_bytes = KP._make_probe(num_blocks, self.shape_tail, self.device, 0)
+        shape = (num_blocks, *self.shape_tail)
+        _capi.check(_capi.lib().mkv_fill_zero(self._v_arena.base + num_blocks * self.block_bytes, self._v_pad,
+                                              _capi.current_stream()))
+        timings = {off: float("inf") for off in KP.CANDIDATE_OFFSETS}
+        for _ in range(3):
+            for off in KP.CANDIDATE_OFFSETS:
+                v = torch.as_tensor(_RawDeviceMemory(self._v_arena.base + off, shape, self._v_arena), device=self.device)
+                timings[off] = min(timings[off], KP._probe_us(self.k_cache, v, probe, layers))
+        best = min(timings, key=timings.get)
+        if timings[best] > 0.995 * timings[0]:
+            best = 0
+        self._v_off = best
+        self._make_views(num_blocks)
+        self.kv_placement = dict(self.kv_placement, v_offset_bytes=best, tuned=True,
+                                 probe_us_per_launch={str(k): round(v, 2) for k, v in timings.items()},
+                                 probe_GBs=round(probe_bytes / timings[best] / 1e3, 1))
 
     def _settle(self, num_blocks: int, settle_seconds: Optional[float]) -> None:
         """``allocate_kv_caches``' one retry for mapped memory: a large pool whose probe reads recycled memory is
@@ -134,7 +172,7 @@ class VmmKVPool(ElasticKVPool):
         torch.cuda.synchronize(self.device)
         self.k_cache = self.v_cache = None
         self._k_arena.resize(0)
-        self._v_arena.resize(0)
+        self._v_arena.resize(0)                              # the extra chunk of a staggered V range included
         time.sleep(settle_seconds)
         self._map(num_blocks)
         self._zero(0, num_blocks)
@@ -147,22 +185,23 @@ class VmmKVPool(ElasticKVPool):
         nbytes = num_blocks * self.block_bytes
         self._k_arena.resize(nbytes)
         try:
-            self._v_arena.resize(nbytes)
+            self._v_arena.resize(nbytes + self._v_pad)
         except Exception:
-            self._k_arena.resize(self._v_arena.mapped_bytes())
+            self._k_arena.resize(max(0, self._v_arena.mapped_bytes() - self._v_pad))
             raise
         self._make_views(num_blocks)
 
     def _make_views(self, num_blocks: int) -> None:
         shape = (num_blocks, *self.shape_tail)
         self.k_cache = torch.as_tensor(_RawDeviceMemory(self._k_arena.base, shape, self._k_arena), device=self.device)
-        self.v_cache = torch.as_tensor(_RawDeviceMemory(self._v_arena.base, shape, self._v_arena), device=self.device)
+        self.v_cache = torch.as_tensor(_RawDeviceMemory(self._v_arena.base + self._v_off, shape, self._v_arena),
+                                       device=self.device)
 
     def _zero(self, first: int, count: int) -> None:
         lib, stream = _capi.lib(), _capi.current_stream()
         off, nbytes = first * self.block_bytes, count * self.block_bytes
         _capi.check(lib.mkv_fill_zero(self._k_arena.base + off, nbytes, stream))
-        _capi.check(lib.mkv_fill_zero(self._v_arena.base + off, nbytes, stream))
+        _capi.check(lib.mkv_fill_zero(self._v_arena.base + self._v_off + off, nbytes, stream))
 
     def descriptor(self) -> _capi.MkvPool:
         return _capi.make_pool(self.k_cache, self.v_cache)

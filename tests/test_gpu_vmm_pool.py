@@ -15,6 +15,20 @@ pytestmark = pytest.mark.gpu
 L, HKV, D, B = 2, 2, 128, 16
 
 
+@pytest.fixture(autouse=True, params=[0, 8192], ids=["plain", "v_staggered"])
+def _v_stagger(request, monkeypatch):
+    """Every test of this file runs twice: with the V tensor at the start of its range and 8 KiB into it (the
+    placement a large pool may choose for itself; it maps one chunk more)."""
+    import morphserve_amd.vmm_pool as VP
+    orig = VP.VmmKVPool.__init__
+
+    def init(self, *a, **k):
+        k.setdefault("v_stagger_bytes", request.param)
+        orig(self, *a, **k)
+    monkeypatch.setattr(VP.VmmKVPool, "__init__", init)
+    return request.param
+
+
 def _i32(x, dev):
     return torch.tensor(list(x), dtype=torch.int32, device=dev)
 
