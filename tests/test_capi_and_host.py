@@ -186,6 +186,11 @@ def test_bad_arguments_are_refused_before_any_launch():
         "mkv_bt_remap": (None, 4, None, 4, None, 8, None),
         "mkv_arena_create": (0, 0, None),
         "mkv_arena_resize": (None, 0),
+        "mkv_arena_move_tail": (None, None, 4096),
+        "mkv_diag_slab_gather/not a power of two": (A, A, 1000, 8, 8, 4, 2, 0, 0, A, None),
+        "mkv_diag_slab_gather/loads in flight": (A, A, 1024, 8, 8, 3, 2, 0, 0, A, None),
+        "mkv_diag_slab_gather/unaligned": (A + 64, A, 1024, 8, 8, 4, 2, 0, 0, A, None),
+        "mkv_diag_slab_gather/workgroups per CU": (A, A, 1024, 8, 8, 4, 9, 0, 0, A, None),
         "mkv_set_decode_variant": (99,),
         "mkv_set_prefill_variant": (5,),
         "mkv_diag_mfma_loop": (7, 1, None, None, None, None),
