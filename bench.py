@@ -365,7 +365,10 @@ def bench_decode(args):
                                  "inside the timed region" if _balanced_order() and getattr(st, "_morphkv_decode_order", None)
                                  else "the grid takes the rows as given (a split batch needs no order)" if _balanced_order()
                                  else "the grid takes the rows as given")
-                                + (", lengths handed over pre-ordered (--seq-order snake)" if args.seq_order == "snake" else "")},
+                                + (", lengths handed over pre-ordered (--seq-order snake)" if args.seq_order == "snake" else ""),
+                   "pool_creation": "outside the timed region; the library's default: a short gather probe picks the V "
+                                    "pool's start and, when it reads memory the driver is still recycling, the pool is "
+                                    "allocated once more after a wait (see kv_placement: v_offset_bytes, probe_GBs, settled)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "kv_placement": kv_placement,
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
