@@ -2,15 +2,22 @@
 
 The library is the only compute path of this package: when it cannot be loaded
 the import of any operator raises; there is no CPU or eager fallback.
+
+``diag_lib()`` loads ``libmorphkv_diag.so``, the diagnostic twin built from the same sources
+(``include/morphkv_diag.h``: kernel-variant switches, per-launch event timing, per-workgroup time
+stamps, calibration loops).  Nothing in this package calls it; benchmarks and tests do, either
+directly or by routing the package's operators through it for a while with ``use_diag_library()``.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
 from typing import Optional, Sequence
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmorphkv.so")
+DIAG_LIB_PATH = os.path.join(_HERE, "csrc", "libmorphkv_diag.so")
 
 MKV_OK, MKV_EINVAL, MKV_EHIP, MKV_ENOSPC, MKV_ELOGIC = 0, -1, -2, -3, -4
 MKV_MAX_SEGMENTS = 128
@@ -60,8 +67,6 @@ PROTOTYPES = {
     "mkv_decode_append_attn": [_P, _P, _P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32, _P, _P, _P],
     "mkv_decode_rope_append_attn": [_P, _P, _P, _P, _P, _P, _PP, _P, _I64, _P, _P, _I32, _I32, _F32, _I32, _I32, _I32,
                                     _P, _P, _P],
-    "mkv_set_decode_variant": [_I32],
-    "mkv_set_prefill_variant": [_I32],
     "mkv_prefill_attn": [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _F32, _P],
     "mkv_prefill_attn_paged": [_P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F32, _I32, _P],
     "mkv_bm_allocate": [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I32, _I32, _P, _I64, _P, _P],
@@ -85,6 +90,11 @@ PROTOTYPES = {
                                _I32, _I32, _I32, _P],
     "mkv_swap_blocks": [_P, _P, _I64, _I32, _PP, _P, _P, C.POINTER(_I64), _P],
     "mkv_swap_blocks_device_ids": [_P, _P, _I64, _I32, _PP, _P, _P, _I64, _P],
+}
+# entries of the diagnostic twin only (include/morphkv_diag.h)
+DIAG_PROTOTYPES = {
+    "mkv_set_decode_variant": [_I32],
+    "mkv_set_prefill_variant": [_I32],
     "mkv_diag_mfma_loop": [_I32, _I32, _P, _P, C.POINTER(C.c_double), _P],
     "mkv_diag_timeline": [_P, _I64],
     "mkv_diag_slab_gather": [_P, _P, _U64, _I32, _I32, _I32, _I32, _I32, C.c_uint32, _P, _P],
@@ -95,6 +105,7 @@ PROTOTYPES = {
 _RESTYPES = {"mkv_last_error": C.c_char_p}
 
 _lib: Optional[C.CDLL] = None
+_diag_lib: Optional[C.CDLL] = None
 
 
 class MorphKVError(RuntimeError):
@@ -105,24 +116,50 @@ class MorphKVError(RuntimeError):
         self.code = code
 
 
+def _load(path: str, prototypes) -> C.CDLL:
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: build it with `python -m morphserve_amd.csrc.build` "
+            "(there is no fallback path)")
+    handle = C.CDLL(path)
+    for name, argtypes in prototypes.items():
+        fn = getattr(handle, name)
+        fn.argtypes = argtypes
+        fn.restype = _RESTYPES.get(name, C.c_int)
+    if handle.mkv_sizeof_pool() != C.sizeof(MkvPool):
+        raise ImportError("mkv_pool layout of the library does not match this binding")
+    return handle
+
+
 def lib() -> C.CDLL:
     """Load the library (once).  Raises when it has not been built."""
     global _lib
     if _lib is None:
         path = os.environ.get("MORPHKV_LIBRARY") or LIB_PATH     # another build of the same ABI, for A/B runs
-        if not os.path.exists(path):
-            raise ImportError(
-                f"{path} is missing: build it with `python -m morphserve_amd.csrc.build` "
-                "(there is no fallback path)")
-        handle = C.CDLL(path)
-        for name, argtypes in PROTOTYPES.items():
-            fn = getattr(handle, name)
-            fn.argtypes = argtypes
-            fn.restype = _RESTYPES.get(name, C.c_int)
-        if handle.mkv_sizeof_pool() != C.sizeof(MkvPool):
-            raise ImportError("mkv_pool layout of the library does not match this binding")
-        _lib = handle
+        _lib = _load(path, PROTOTYPES)
     return _lib
+
+
+def diag_lib() -> C.CDLL:
+    """Load the diagnostic twin (once): every entry of ``lib()`` plus ``DIAG_PROTOTYPES``."""
+    global _diag_lib
+    if _diag_lib is None:
+        _diag_lib = _load(os.environ.get("MORPHKV_DIAG_LIBRARY") or DIAG_LIB_PATH,
+                          {**PROTOTYPES, **DIAG_PROTOTYPES})
+    return _diag_lib
+
+
+@contextlib.contextmanager
+def use_diag_library():
+    """Route every call of this package through the diagnostic twin inside the ``with`` block
+    (measurement and tests; process-wide, so not while other threads are issuing calls)."""
+    global _lib
+    lib()
+    saved, _lib = _lib, diag_lib()
+    try:
+        yield _lib
+    finally:
+        _lib = saved
 
 
 def check(rc: int) -> None:
@@ -133,6 +170,25 @@ def check(rc: int) -> None:
 def current_stream() -> int:
     import torch
     return torch.cuda.current_stream().cuda_stream
+
+
+_hip_runtime = None
+
+
+def capture_id(stream: int) -> Optional[int]:
+    """Id of the graph capture ``stream`` is recording into, ``None`` when it is not capturing
+    (``hipStreamGetCaptureInfo`` of the HIP runtime torch has already loaded)."""
+    global _hip_runtime
+    if _hip_runtime is None:
+        _hip_runtime = C.CDLL("libamdhip64.so")
+        _hip_runtime.hipStreamGetCaptureInfo.argtypes = [_P, C.POINTER(C.c_int), C.POINTER(C.c_ulonglong)]
+        _hip_runtime.hipStreamGetCaptureInfo.restype = C.c_int
+    status = C.c_int(0)
+    cid = C.c_ulonglong(0)
+    rc = _hip_runtime.hipStreamGetCaptureInfo(stream, C.byref(status), C.byref(cid))
+    if rc != 0:
+        raise MorphKVError(MKV_EHIP, f"hipStreamGetCaptureInfo failed with HIP error {rc}")
+    return int(cid.value) if status.value == 1 else None      # 1 = hipStreamCaptureStatusActive
 
 
 def ptr(t) -> int:
@@ -162,16 +218,17 @@ def make_pool(k_cache, v_cache, k_segments: Sequence = (), v_segments: Sequence 
 
 
 def prof_enable(on: bool) -> None:
-    check(lib().mkv_prof_enable(1 if on else 0))
+    """Per-launch event timing of the DIAGNOSTIC twin (calls must go through it: ``use_diag_library()``)."""
+    check(diag_lib().mkv_prof_enable(1 if on else 0))
 
 
 def prof_reset() -> None:
-    check(lib().mkv_prof_reset())
+    check(diag_lib().mkv_prof_reset())
 
 
 def prof_collect(kernel_id: int):
     """(launches, total_ms) of one instrumented kernel since the last reset."""
     n = _I64(0)
     ms = C.c_double(0.0)
-    check(lib().mkv_prof_collect(kernel_id, C.byref(n), C.byref(ms)))
+    check(diag_lib().mkv_prof_collect(kernel_id, C.byref(n), C.byref(ms)))
     return n.value, ms.value

@@ -7,7 +7,17 @@
 #include <stdio.h>
 
 #include "morphkv.h"
+
+// MKV_DIAG = 1 builds the diagnostic twin of the library (libmorphkv_diag.so): the same entry points plus
+// the switches and measurement hooks of morphkv_diag.h.  The product library is built with MKV_DIAG = 0 and
+// carries none of them: no time-stamp argument in any kernel, no event pairs around launches, no process-wide
+// variant switches.
+#ifndef MKV_DIAG
+#define MKV_DIAG 0
+#endif
+#if MKV_DIAG
 #include "morphkv_diag.h"
+#endif
 
 namespace mkv {
 
@@ -31,7 +41,11 @@ int  hip_fail(hipError_t e, const char* what);
 
 int  check_pool(const mkv_pool* p);
 
-// Brackets one launch with an event pair when profiling is on.
+// Number of compute units of the current device (cached per process; 256 when the query fails).
+int num_cus();
+
+#if MKV_DIAG
+// Brackets one launch with an event pair when profiling is on (diagnostic build only).
 struct ProfScope {
     int kernel_id;
     hipStream_t stream;
@@ -39,6 +53,10 @@ struct ProfScope {
     ProfScope(int kernel_id, hipStream_t s);
     ~ProfScope();
 };
+#define MKV_PROF(id, s) ::mkv::ProfScope mkv_prof_scope_((id), (s))
+#else
+#define MKV_PROF(id, s) do { } while (0)
+#endif
 
 // ---- device-side pool addressing ---------------------------------------------
 // Byte offset of a block inside its pool/segment and the K/V bases it is
@@ -76,19 +94,31 @@ __host__ __device__ __forceinline__ int64_t pool_total_blocks(const mkv_pool& p)
 
 static inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
-// ---- per-workgroup time stamps (diagnostic, mkv_diag_timeline) -----------------
-// The attention launchers hand their kernels the buffer set by mkv_diag_timeline when it holds the
-// launch's workgroups, NULL otherwise.  With a buffer, thread 0 of workgroup w stores the constant-rate
-// 100 MHz counter at point k of its life into buf[w * MKV_TIMELINE_POINTS + k]; without one a mark is
-// a scalar test and a branch.
+// ---- per-workgroup time stamps (diagnostic build only, mkv_diag_timeline) --------
+// The attention kernels take a TimelineArg<TL> as their last argument.  TL = false, the only instance the
+// product library contains, is an empty struct whose mark() is nothing.  In the diagnostic build the
+// launchers pick the TL = true instance while mkv_diag_timeline holds a buffer large enough for the
+// launch's workgroups: thread 0 of workgroup w then stores the constant-rate 100 MHz counter at point k
+// of its life into buf[w * MKV_TIMELINE_POINTS + k].
+template <bool TL>
+struct TimelineArg {
+    __device__ __forceinline__ void mark(int64_t, int) const {}
+};
+
+#if MKV_DIAG
 long long* timeline_buffer(int64_t workgroups);
 
-__device__ __forceinline__ void timeline_mark(long long* tl, int64_t wg, int k) {
-    if (tl != nullptr && threadIdx.x == 0) {
-        unsigned long long t;
-        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t));
-        tl[wg * MKV_TIMELINE_POINTS + k] = (long long)t;
+template <>
+struct TimelineArg<true> {
+    long long* buf;
+    __device__ __forceinline__ void mark(int64_t wg, int k) const {
+        if (threadIdx.x == 0) {
+            unsigned long long t;
+            asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t));
+            buf[wg * MKV_TIMELINE_POINTS + k] = (long long)t;
+        }
     }
-}
+};
+#endif
 
 }  // namespace mkv

@@ -48,6 +48,19 @@ int check_pool(const mkv_pool* p) {
     return MKV_OK;
 }
 
+int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+#if MKV_DIAG
 // ---- per-workgroup time stamps -----------------------------------------------------
 static long long* g_timeline = nullptr;
 static int64_t g_timeline_wgs = 0;
@@ -83,6 +96,7 @@ ProfScope::~ProfScope() {
     g_prof[kernel_id].push_back(*r);
     delete r;
 }
+#endif  // MKV_DIAG
 
 }  // namespace mkv
 
@@ -111,6 +125,7 @@ int mkv_pool_set_strided(mkv_pool* pool, void* k_new0, void* v_new0,
     return MKV_OK;
 }
 
+#if MKV_DIAG
 int mkv_diag_timeline(void* buf, int64_t max_workgroups) {
     MKV_REQUIRE(buf == nullptr || max_workgroups > 0, "max_workgroups must be positive with a buffer");
     MKV_REQUIRE(((uintptr_t)buf & 7) == 0, "the time stamp buffer must be 8-byte aligned");
@@ -152,5 +167,6 @@ int mkv_prof_collect(int32_t kernel_id, int64_t* launches, double* total_ms) {
     *total_ms = sum;
     return MKV_OK;
 }
+#endif  // MKV_DIAG
 
 }  // extern "C"

@@ -127,7 +127,7 @@ int mkv_append_decode(const void* k, const void* v, const mkv_pool* pool,
     const int64_t blocks = (total + threads - 1) / threads;
     hipStream_t s = (hipStream_t)stream;
     {
-        mkv::ProfScope prof(MKV_K_APPEND_DECODE, s);
+        MKV_PROF(MKV_K_APPEND_DECODE, s);
         hipLaunchKernelGGL(mkv::append_decode_kernel, dim3((unsigned)blocks), dim3(threads), 0, s,
                            (const uint4*)k, (const uint4*)v, *pool, block_table, max_blocks_per_seq,
                            seq_ids, seq_lens, n, layer);
@@ -161,7 +161,7 @@ int mkv_append_prefill(const void* k, const void* v, const mkv_pool* pool,
               2u * (unsigned)mkv::cdiv(pool->num_kv_heads, heads_per_part));
     hipStream_t s = (hipStream_t)stream;
     {
-        mkv::ProfScope prof(MKV_K_APPEND_PREFILL, s);
+        MKV_PROF(MKV_K_APPEND_PREFILL, s);
         hipLaunchKernelGGL(mkv::append_prefill_kernel, grid, dim3(256), 0, s, (const uint4*)k,
                            (const uint4*)v, *pool, block_table, max_blocks_per_seq, seq_ids,
                            start_locs, seq_lens, layer, heads_per_part);

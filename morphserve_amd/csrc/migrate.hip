@@ -104,18 +104,6 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, i
     if (blockIdx.x == 0 && (int)threadIdx.x < tail_bytes) tail[threadIdx.x] = 0;
 }
 
-static int num_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
-    return cus;
-}
-
 }  // namespace mkv
 
 extern "C" {
@@ -134,7 +122,7 @@ int mkv_pool_migrate(const mkv_pool* pool, const int64_t* src, const int64_t* ds
     const unsigned grid = (unsigned)(items < want ? items : want);
     hipStream_t s = (hipStream_t)stream;
     {
-        mkv::ProfScope prof(MKV_K_MIGRATE, s);
+        MKV_PROF(MKV_K_MIGRATE, s);
         hipLaunchKernelGGL(mkv::pool_migrate_kernel, dim3(grid), dim3(mkv::kCopyThreads), 0, s,
                            *pool, src, dst, num_moves, block_bytes, chunks);
     }
@@ -156,7 +144,7 @@ int mkv_fill_zero(void* ptr, uint64_t bytes, void* stream) {
         const int tail = (int)(now & 15);
         const int64_t grid = units > 0 ? (units + 255) / 256 : 1;
         {
-            mkv::ProfScope prof(MKV_K_FILL_ZERO, s);
+            MKV_PROF(MKV_K_FILL_ZERO, s);
             hipLaunchKernelGGL(mkv::fill_zero_kernel, dim3((unsigned)grid), dim3(256), 0, s, (uint4*)cur,
                                units, (uint8_t*)cur + (units << 4), tail);
         }
@@ -256,7 +244,7 @@ int mkv_swap_blocks_device_ids(const int64_t* src_ids, const int64_t* dst_ids, i
     const unsigned grid = (unsigned)(items < want ? items : want);
     hipStream_t s = (hipStream_t)stream;
     {
-        mkv::ProfScope prof(MKV_K_SWAP, s);
+        MKV_PROF(MKV_K_SWAP, s);
         if (is_swap_in) {
             hipLaunchKernelGGL(mkv::pool_swap_kernel<true>, dim3(grid), dim3(mkv::kCopyThreads), 0, s, *pool,
                                src_ids, dst_ids, count, (char*)dev_ptr[0], (char*)dev_ptr[1], num_host_blocks,

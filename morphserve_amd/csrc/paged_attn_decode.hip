@@ -169,7 +169,7 @@ __global__ __launch_bounds__(1024) void decode_order_kernel(const int32_t* __res
     }
 }
 
-template <int G>
+template <int G, bool TL>
 __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ q,        // [n, Hq, D] fp16
     __half* __restrict__ o,             // [n, Hq, D] fp16 (written only when gridDim.x == 1)
@@ -183,16 +183,19 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     const uint4* __restrict__ cos_t,    // [n, D/2] fp16 or NULL: rotate q and the new k row on the way in
     const uint4* __restrict__ sin_t,
     const int32_t* __restrict__ order,     // [n] or NULL: batch row taken by each slot of the grid
-    long long* __restrict__ timeline) {    // per-workgroup time stamps (diagnostic) or NULL
+    const TimelineArg<TL> timeline) {      // per-workgroup time stamps (an empty struct unless TL)
     const int64_t wg_id = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-    timeline_mark(timeline, wg_id, 0);
+    timeline.mark(wg_id, 0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int r = lane >> 4;       // token row within a group of four
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
-    const int i = order ? order[blockIdx.z] : (int)blockIdx.z;
+    // a slot's row comes from the caller's order; an entry outside the batch (a buffer that was never
+    // written) falls back to the slot's own row instead of indexing past the batch's arrays
+    int i = order ? order[blockIdx.z] : (int)blockIdx.z;
+    if ((unsigned)i >= gridDim.z) i = (int)blockIdx.z;
     const int Hq = pool.num_kv_heads * G;
 
     const int len = seq_lens[i];
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     // is handled apart, so the main loop carries no masking and no branches around
     // its loads: the loads of block t+1 are issued before block t is consumed and
     // stay in flight behind it.
-    timeline_mark(timeline, wg_id, 1);
+    timeline.mark(wg_id, 1);
     const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
     const int n_it = max(0, (blk_end - my_first + 3) >> 2);
     // blocks [0, nblk_full) hold 16 valid tokens and need no special care; with a
@@ -361,7 +364,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     }
 
     // ---- merge the four waves through LDS ------------------------------------------
-    timeline_mark(timeline, wg_id, 2);
+    timeline.mark(wg_id, 2);
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
     __shared__ float sm_l[4][G];
@@ -379,7 +382,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1(
     __syncthreads();
     merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
                              max_splits);
-    timeline_mark(timeline, wg_id, 3);
+    timeline.mark(wg_id, 3);
 }
 
 // ---- matrix-core variant for GQA groups (G >= 4) -----------------------------------
@@ -410,7 +413,7 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int G>
+template <int G, bool TL>
 __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     const uint4* __restrict__ q, __half* __restrict__ o, float* __restrict__ mid_o,
     float* __restrict__ mid_lse, const mkv_pool pool, const int32_t* __restrict__ block_table,
@@ -418,9 +421,9 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     const int32_t* __restrict__ seq_lens, float scale2, int32_t layer, int32_t blocks_per_split,
     int32_t max_splits, const uint4* __restrict__ k_new, const uint4* __restrict__ v_new,
     const uint4* __restrict__ cos_t, const uint4* __restrict__ sin_t, const int32_t* __restrict__ order,
-    long long* __restrict__ timeline) {
+    const TimelineArg<TL> timeline) {
     const int64_t wg_id = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-    timeline_mark(timeline, wg_id, 0);
+    timeline.mark(wg_id, 0);
     __shared__ __attribute__((aligned(16))) char stage[4][2][kLdsTile];
     __shared__ float sm_acc[4][G][kD];
     __shared__ float sm_m[4][G];
@@ -433,7 +436,10 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     const int c = lane >> 4;       // lane group
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
-    const int i = order ? order[blockIdx.z] : (int)blockIdx.z;
+    // a slot's row comes from the caller's order; an entry outside the batch (a buffer that was never
+    // written) falls back to the slot's own row instead of indexing past the batch's arrays
+    int i = order ? order[blockIdx.z] : (int)blockIdx.z;
+    if ((unsigned)i >= gridDim.z) i = (int)blockIdx.z;
     const int Hq = pool.num_kv_heads * G;
 
     const int len = seq_lens[i];
@@ -578,7 +584,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         wave_lds_fence();                            // reads done before the next tile is staged
     };
 
-    timeline_mark(timeline, wg_id, 1);
+    timeline.mark(wg_id, 1);
     const int my_first = blk_begin + __builtin_amdgcn_readfirstlane(wave);
     const int n_it = max(0, (blk_end - my_first + 3) >> 2);
     // blocks [0, nblk_full) hold 16 valid tokens; the final block takes the careful
@@ -623,7 +629,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
         }
     }
 
-    timeline_mark(timeline, wg_id, 2);
+    timeline.mark(wg_id, 2);
     float l_tot = l_run + __shfl_xor(l_run, 16);
     l_tot += __shfl_xor(l_tot, 32);
     if (n < G) {
@@ -639,7 +645,7 @@ __global__ __launch_bounds__(256) void attn_decode_phase1_mfma(
     __syncthreads();
     merge_waves_and_store<G>(sm_acc, sm_m, sm_l, o, mid_o, mid_lse, (int64_t)i * Hq + kvh * G, split,
                              max_splits);
-    timeline_mark(timeline, wg_id, 3);
+    timeline.mark(wg_id, 3);
 }
 
 // Phase 2: log-sum-exp merge of the per-split partials, cast to fp16.  Both kernels read
@@ -738,8 +744,41 @@ __global__ __launch_bounds__(256) void attn_decode_phase2_wide(
     }
 }
 
-// 0: by group size (matrix cores for G >= 4), 1: vector ALU kernel, 2: matrix-core kernel
+#if MKV_DIAG
+// 0: by group size (matrix cores for G >= 3), 1: vector ALU kernel, 2: matrix-core kernel
 static int g_decode_variant = 0;
+#endif
+
+template <int G, bool TL>
+static void launch_phase1_as(bool mfma, dim3 grid, hipStream_t s, const void* q, void* o, void* mid_o,
+                             void* mid_lse, const mkv_pool* pool, const int32_t* block_table,
+                             int64_t max_blocks_per_seq, const int32_t* seq_ids, const int32_t* seq_lens,
+                             float scale2, int32_t layer, int32_t blocks_per_split, int32_t max_splits,
+                             const void* k_new, const void* v_new, const void* cos_t, const void* sin_t,
+                             const int32_t* order, const TimelineArg<TL> timeline) {
+    // The vector-ALU kernel serves one or two q heads per kv head, the matrix-core kernel every larger
+    // group (up to the 16 columns of a matrix tile).  The diagnostic build also holds the vector kernel
+    // for groups of 4 and 8 and the matrix kernel for 1 and 2, for A/B runs.
+    constexpr bool valu_built = MKV_DIAG ? (G == 1 || G == 2 || G == 4 || G == 8) : (G <= 2);
+    constexpr bool mfma_built = MKV_DIAG ? true : (G >= 3);
+    if constexpr (mfma_built) {
+        if (mfma || !valu_built) {
+            hipLaunchKernelGGL((attn_decode_phase1_mfma<G, TL>), grid, dim3(256), 0, s, (const uint4*)q,
+                               (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
+                               max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
+                               max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
+                               (const uint4*)sin_t, order, timeline);
+            return;
+        }
+    }
+    if constexpr (valu_built) {
+        hipLaunchKernelGGL((attn_decode_phase1<G, TL>), grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
+                           (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
+                           seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
+                           (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t,
+                           order, timeline);
+    }
+}
 
 template <int G>
 static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void* mid_o,
@@ -748,35 +787,36 @@ static void launch_phase1(dim3 grid, hipStream_t s, const void* q, void* o, void
                           const int32_t* seq_lens, float scale2, int32_t layer,
                           int32_t blocks_per_split, int32_t max_splits, const void* k_new,
                           const void* v_new, const void* cos_t, const void* sin_t, const int32_t* order) {
-    // the vector-ALU kernel exists for the power-of-two groups only; every other group
-    // size (up to the 16 columns of a matrix tile) runs on the matrix cores
-    constexpr bool has_valu = G == 1 || G == 2 || G == 4 || G == 8;
-    const bool mfma = !has_valu || g_decode_variant == 2 || (g_decode_variant == 0 && G >= 4);
-    long long* timeline = timeline_buffer((int64_t)grid.x * grid.y * grid.z);
-    if (mfma) {
-        hipLaunchKernelGGL(attn_decode_phase1_mfma<G>, grid, dim3(256), 0, s, (const uint4*)q,
-                           (__half*)o, (float*)mid_o, (float*)mid_lse, *pool, block_table,
-                           max_blocks_per_seq, seq_ids, seq_lens, scale2, layer, blocks_per_split,
-                           max_splits, (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t,
-                           (const uint4*)sin_t, order, timeline);
-    } else if constexpr (has_valu) {
-        hipLaunchKernelGGL(attn_decode_phase1<G>, grid, dim3(256), 0, s, (const uint4*)q, (__half*)o,
-                           (float*)mid_o, (float*)mid_lse, *pool, block_table, max_blocks_per_seq,
-                           seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits,
-                           (const uint4*)k_new, (const uint4*)v_new, (const uint4*)cos_t, (const uint4*)sin_t,
-                           order, timeline);
+    bool mfma = G >= 3;
+#if MKV_DIAG
+    if (g_decode_variant == 1) mfma = false;
+    if (g_decode_variant == 2) mfma = true;
+    // time stamps: the groups the timeline workloads use
+    if constexpr (G == 1 || G == 2 || G == 4 || G == 8) {
+        if (long long* buf = timeline_buffer((int64_t)grid.x * grid.y * grid.z)) {
+            launch_phase1_as<G, true>(mfma, grid, s, q, o, mid_o, mid_lse, pool, block_table, max_blocks_per_seq,
+                                      seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits, k_new, v_new,
+                                      cos_t, sin_t, order, TimelineArg<true>{buf});
+            return;
+        }
     }
+#endif
+    launch_phase1_as<G, false>(mfma, grid, s, q, o, mid_o, mid_lse, pool, block_table, max_blocks_per_seq,
+                               seq_ids, seq_lens, scale2, layer, blocks_per_split, max_splits, k_new, v_new,
+                               cos_t, sin_t, order, TimelineArg<false>{});
 }
 
 }  // namespace mkv
 
 extern "C" {
 
+#if MKV_DIAG
 int mkv_set_decode_variant(int32_t variant) {
     MKV_REQUIRE(variant >= 0 && variant <= 2, "variant must be 0 (auto), 1 (vector ALU) or 2 (matrix core)");
     mkv::g_decode_variant = variant;
     return MKV_OK;
 }
+#endif
 
 int mkv_paged_attn_scratch_bytes(int32_t n, int32_t num_q_heads, int32_t head_dim,
                                  int32_t max_splits, int64_t* mid_o_bytes,
@@ -817,7 +857,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)max_splits, (unsigned)pool->num_kv_heads, (unsigned)n);
     {
-        mkv::ProfScope prof(MKV_K_ATTN_PHASE1, s);
+        MKV_PROF(MKV_K_ATTN_PHASE1, s);
         switch (G) {
 #define MKV_CASE(GG)                                                                               \
     case GG:                                                                                       \
@@ -849,7 +889,7 @@ static int decode_impl(const void* q, void* o, const mkv_pool* pool, const int32
     }
     MKV_HIP(hipGetLastError());
     if (max_splits > 1) {
-        mkv::ProfScope prof(MKV_K_ATTN_PHASE2, s);
+        MKV_PROF(MKV_K_ATTN_PHASE2, s);
         if (max_splits > 8) {       // a long chain of partials per head: the gather-in-parallel merge
             hipLaunchKernelGGL(mkv::attn_decode_phase2_wide, dim3((unsigned)num_q_heads, (unsigned)n),
                                dim3(256), 0, s, (const float*)mid_o, (const float*)mid_lse, (__half*)o,
@@ -957,9 +997,10 @@ int mkv_decode_order(const int32_t* seq_lens, int32_t n, int32_t num_kv_heads, i
     MKV_REQUIRE(seq_lens && order, "NULL argument");
     MKV_REQUIRE(n <= 4096, "at most 4096 sequences (got %d)", n);
     MKV_REQUIRE(num_kv_heads > 0, "num_kv_heads must be positive");
-    // slots one run apart share a CU (256 CUs, one workgroup per kv head and slot); when the kv heads do
-    // not divide the CU count there is no such pairing and the order is plain longest-first
-    const int run = (256 % num_kv_heads == 0 && 256 / num_kv_heads >= 1) ? 256 / num_kv_heads : n;
+    // slots one run apart share a CU (one workgroup per kv head and slot, handed to the CUs in turn); when
+    // the kv heads do not divide the CU count there is no such pairing and the order is plain longest-first
+    const int cus = mkv::num_cus();
+    const int run = (cus % num_kv_heads == 0 && cus / num_kv_heads >= 1) ? cus / num_kv_heads : n;
     hipLaunchKernelGGL(mkv::decode_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seq_lens, n, run, order);
     MKV_HIP(hipGetLastError());
     return MKV_OK;

@@ -71,7 +71,6 @@ struct PrefillArgs {
     int32_t num_seqs;
     int32_t num_q_tiles;          // ceil(max_len / query rows per workgroup)
     int32_t pair_tiles;           // 1: a workgroup takes two query tiles (i-th from the end, i-th from the start); 0: one
-    long long* timeline;          // per-workgroup time stamps (diagnostic) or NULL
 };
 
 __device__ __forceinline__ float pf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -92,9 +91,11 @@ __device__ __forceinline__ float max_over_groups(float x) {
     auto b = __builtin_amdgcn_permlane32_swap(yi, yi, false, false);
     return fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
 }
-// TL: the instance that takes per-workgroup time stamps (launched only while mkv_diag_timeline holds a buffer)
+// TL: the instance that takes per-workgroup time stamps (diagnostic build only, launched while mkv_diag_timeline
+// holds a buffer); the product library holds the TL = false instances alone
 template <bool PAGED, int WAVES, bool TL>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool) {
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attn_kernel(const PrefillArgs a, const mkv_pool pool,
+                                                                                                    const TimelineArg<TL> timeline) {
     constexpr int kThreads = 64 * WAVES;
     constexpr int kQTile = 16 * kU * WAVES;                    // query rows per workgroup
     constexpr int kFetchSteps = (kKTile * 16) / kThreads;      // 16-byte units per thread per K (or V) tile
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     __shared__ __attribute__((aligned(16))) char v_lds[2 * kVBuf];
 
     const int tid = threadIdx.x;
-    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 0);
+    timeline.mark(blockIdx.x, 0);
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int m = lane & 15;          // query row of a column tile (B / C), key or dim row (A)
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         __syncthreads();
     }
     carried = false;
-    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 1 + 3 * part);
+    timeline.mark(blockIdx.x, 1 + 3 * part);
     for (int it = 0; it + 1 < num_tiles; it += 2) {
         iteration(it, Set0{}, Set1{});
         if (it + 2 < num_tiles) iteration(it + 1, Set1{}, Set0{});
@@ -494,7 +495,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         }
         __syncthreads();                              // every read of the staged tiles is done
     }
-    if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 2 + 3 * part);
+    timeline.mark(blockIdx.x, 2 + 3 * part);
 
     // Output: a lane holds four dims of sixteen rows' worth of 8-byte pieces; the column tile goes
     // through this wave's corner of the idle V buffer (rows 288 bytes apart: conflict-free 8-byte
@@ -523,7 +524,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         if (more) stage_tile(0, Set0{});
         if (follows) __syncthreads();                 // the next part's staging may reuse every buffer
         if (more) carried = true;
-        if constexpr (TL) timeline_mark(a.timeline, blockIdx.x, 3 + 3 * part);
+        timeline.mark(blockIdx.x, 3 + 3 * part);
     }
   }   // part
 }
@@ -531,8 +532,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 static constexpr int kLongPrompt = 2048;    // shortest prompt (or chunk) from which the eight-wave kernel is used
 static constexpr int kChunkRows = 256;      // ... or a chunk of at least this many rows (one eight-wave query tile)
 static constexpr int kLongPrefix = 512;     //     over a cached prefix of at least this many tokens
+#if MKV_DIAG
 static int g_prefill_waves = 0;             // 0: by length; 4 or 8: forced (experiments and tests)
 static int g_prefill_pairing = 0;           // 0: by grid size; 1: always two tiles per workgroup; 2: never
+#else
+static constexpr int g_prefill_waves = 0;   // the product library always chooses by the call
+static constexpr int g_prefill_pairing = 0;
+#endif
 
 static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool, int num_seqs,
                           int max_len, int max_prefix, hipStream_t s) {
@@ -546,7 +552,8 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
                            (max_len >= kChunkRows && max_prefix >= kLongPrefix && max_len + max_prefix >= 1024);
     // (over the batch's own k, v a grid of exactly one eight-wave workgroup per CU loses to two four-wave ones:
     // 2 x 2048 tokens 86 against 79 us, 1 x 4096 158 against 142 us; from one and a half per CU on it wins)
-    const bool long_and_wide = many_keys && pairs8 * ((cdiv(max_len, 16 * kU * 8) + 1) / 2) >= (paged ? 256 : 320);
+    const int cus = num_cus();
+    const bool long_and_wide = many_keys && pairs8 * ((cdiv(max_len, 16 * kU * 8) + 1) / 2) >= (paged ? cus : cus + cus / 4);
     const int waves = (g_prefill_waves == 4 || g_prefill_waves == 8) ? g_prefill_waves : (long_and_wide ? 8 : 4);
     const int q_tile = 16 * kU * waves;
     args.num_q_tiles = cdiv(max_len, q_tile);
@@ -555,26 +562,31 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
     // with one tile per workgroup and the balance made across the two workgroups of a CU
     // (4 x 512: 25.7 -> 22.4 us, 3 x 700: 39.0 -> 26.1 us, 1 x 1024: 32.5 -> 27.2 us, 8 x 256: 22.0 -> 18.9 us)
     const int64_t paired = pairs8 * ((args.num_q_tiles + 1) / 2);
-    const bool unpair = paired < 512 || args.num_q_tiles <= 3;
+    const bool unpair = paired < 2 * cus || args.num_q_tiles <= 3;
     args.pair_tiles = (g_prefill_pairing == 1 || (g_prefill_pairing == 0 && !unpair)) ? 1 : 0;
     const int64_t unpaired = ((pairs8 / 8 * args.num_q_tiles + 31) / 32 * 32) * 8;      // whole runs of 32 slots per XCD
     dim3 grid((unsigned)(args.pair_tiles ? paired : unpaired));
-    args.timeline = timeline_buffer(grid.x);
     static const mkv_pool empty = {};
     {
-        ProfScope prof(MKV_K_PREFILL_ATTN, s);
-        const bool tl = args.timeline != nullptr;
-#define MKV_LAUNCH(P, W, T, TH, PL) \
-    hipLaunchKernelGGL((prefill_attn_kernel<P, W, T>), grid, dim3(TH), 0, s, args, PL)
-        if (paged && waves == 8) {
-            if (tl) MKV_LAUNCH(true, 8, true, 512, *pool); else MKV_LAUNCH(true, 8, false, 512, *pool);
-        } else if (paged) {
-            if (tl) MKV_LAUNCH(true, 4, true, 256, *pool); else MKV_LAUNCH(true, 4, false, 256, *pool);
-        } else if (waves == 8) {
-            if (tl) MKV_LAUNCH(false, 8, true, 512, empty); else MKV_LAUNCH(false, 8, false, 512, empty);
-        } else {
-            if (tl) MKV_LAUNCH(false, 4, true, 256, empty); else MKV_LAUNCH(false, 4, false, 256, empty);
+        MKV_PROF(MKV_K_PREFILL_ATTN, s);
+#define MKV_LAUNCH(P, W, T, TH, PL, TA) \
+    hipLaunchKernelGGL((prefill_attn_kernel<P, W, T>), grid, dim3(TH), 0, s, args, PL, TA)
+#if MKV_DIAG
+        if (long long* buf = timeline_buffer(grid.x)) {
+            const TimelineArg<true> ta{buf};
+            if (paged && waves == 8) MKV_LAUNCH(true, 8, true, 512, *pool, ta);
+            else if (paged) MKV_LAUNCH(true, 4, true, 256, *pool, ta);
+            else if (waves == 8) MKV_LAUNCH(false, 8, true, 512, empty, ta);
+            else MKV_LAUNCH(false, 4, true, 256, empty, ta);
+            MKV_HIP(hipGetLastError());
+            return MKV_OK;
         }
+#endif
+        const TimelineArg<false> none{};
+        if (paged && waves == 8) MKV_LAUNCH(true, 8, false, 512, *pool, none);
+        else if (paged) MKV_LAUNCH(true, 4, false, 256, *pool, none);
+        else if (waves == 8) MKV_LAUNCH(false, 8, false, 512, empty, none);
+        else MKV_LAUNCH(false, 4, false, 256, empty, none);
 #undef MKV_LAUNCH
     }
     MKV_HIP(hipGetLastError());
@@ -585,6 +597,7 @@ static int launch_prefill(bool paged, const PrefillArgs& a, const mkv_pool* pool
 
 extern "C" {
 
+#if MKV_DIAG
 int mkv_set_prefill_variant(int32_t waves) {
     const int pairing = (waves >> 8) & 3;       // bits 8-9: 0 tiles paired by grid size, 1 always, 2 never
     waves &= 0xFF;
@@ -593,6 +606,7 @@ int mkv_set_prefill_variant(int32_t waves) {
     mkv::g_prefill_pairing = pairing;
     return MKV_OK;
 }
+#endif
 
 int mkv_prefill_attn(const void* q, const void* k, const void* v, void* o,
                      const int32_t* start_locs, const int32_t* seq_lens, int32_t num_seqs,

@@ -167,7 +167,7 @@ int mkv_rope_store_kvcache(void* q, void* k, const void* v, const void* cos_tabl
     a.decoding_seq_lens = decoding_seq_lens;
     a.layer = layer;
     {
-        mkv::ProfScope prof(MKV_K_ROPE_STORE, s);
+        MKV_PROF(MKV_K_ROPE_STORE, s);
         hipLaunchKernelGGL(mkv::rope_store_kernel<true>, dim3((unsigned)T), dim3(256), 0, s, a, *pool);
     }
     MKV_HIP(hipGetLastError());

@@ -7,7 +7,8 @@ from __future__ import annotations
 
 import ctypes as C
 import os
-from typing import Dict, List, Optional, Tuple
+from collections import OrderedDict
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -18,25 +19,45 @@ from ._pool import pool_from_args
 # Scratch for the per-split partials, grown on demand and reused across calls
 # (the reference allocates it on every call, paged_attn.py:780-793).  One buffer per
 # (device, stream): calls on one stream are ordered, calls on different streams may overlap.
-_scratch: Dict[Tuple[int, int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+# At most MAX_SCRATCH_BUFFERS are kept; the least recently used one is dropped (its memory goes
+# back to torch's allocator, which keeps it valid for work already queued on its stream).
+MAX_SCRATCH_BUFFERS = 8
+_scratch: "OrderedDict[Tuple[int, int, int], Tuple[torch.Tensor, torch.Tensor]]" = OrderedDict()
 
 # "auto": split length chosen here for the MI355X grid; "reference": use the
 # caller's infer_state.seq_block_size as the reference kernels do.
 SPLIT_POLICY = os.environ.get("MORPHKV_SPLIT_POLICY", "auto")
-TARGET_WORKGROUPS = int(os.environ.get("MORPHKV_TARGET_WGS", "512"))
+# Workgroups a decode launch should hold: None = two per compute unit of the device (512 on an
+# MI355X); a number here or in the environment overrides that.
+TARGET_WORKGROUPS: Optional[int] = (int(os.environ["MORPHKV_TARGET_WGS"])
+                                    if os.environ.get("MORPHKV_TARGET_WGS") else None)
+_target_wgs_by_device = {}
 # The grid takes the batch rows in an order that gives every CU about the same number of tokens
 # (``mkv_decode_order``); "0" keeps the rows' own order.
 BALANCED_ORDER = os.environ.get("MORPHKV_DECODE_ORDER", "1") != "0"
 
 
+def target_workgroups(device=None) -> int:
+    if TARGET_WORKGROUPS is not None:
+        return int(TARGET_WORKGROUPS)
+    if not torch.cuda.is_available():
+        return 512                      # host-only use (tests of the split arithmetic): an MI355X's figure
+    idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    wgs = _target_wgs_by_device.get(idx)
+    if wgs is None:
+        wgs = 2 * torch.cuda.get_device_properties(idx).multi_processor_count
+        _target_wgs_by_device[idx] = wgs
+    return wgs
+
+
 def choose_split(n: int, num_kv_heads: int, max_len: int, block_size: int,
                  target_wgs: Optional[int] = None) -> Tuple[int, int]:
     """``(tokens_per_split, max_splits)``: enough (split, kv head, sequence)
-    workgroups to put two on each of the 256 compute units, and no more: every
+    workgroups to put two on each compute unit of the device, and no more: every
     extra split costs a partial write and the phase-2 launch, and a sequence that
     is not split at all is written straight to ``o``.  Each split is a multiple
     of four blocks (one per wave) and never shorter than 128 tokens."""
-    target = TARGET_WORKGROUPS if target_wgs is None else target_wgs
+    target = target_workgroups() if target_wgs is None else target_wgs
     unit = 4 * block_size
     max_len = max(int(max_len), 1)
     want = max(1, -(-target // max(1, n * num_kv_heads)))
@@ -56,6 +77,9 @@ def _get_scratch(device: torch.device, n: int, hq: int, splits: int, d: int):
         cur = (torch.empty(grow * d, dtype=torch.float32, device=device),
                torch.empty(grow, dtype=torch.float32, device=device))
         _scratch[key] = cur
+        while len(_scratch) > MAX_SCRATCH_BUFFERS:
+            _scratch.popitem(last=False)
+    _scratch.move_to_end(key)
     return cur
 
 
@@ -64,26 +88,30 @@ def _decode_order(infer_state, lens: torch.Tensor, n: int, num_kv_heads: int, sp
     for it and kept on ``infer_state`` for the other layers of the step (it depends on the lengths only).
     An order that has gone stale -- lengths updated in place -- is still a permutation, so the outputs
     do not depend on it; only the balance does.  A batch that is cut into splits needs none: its workgroups
-    carry equal token counts already."""
+    carry equal token counts already.
+
+    An order whose launch was only RECORDED into a graph holds nothing until that graph runs, so an
+    entry made during a stream capture serves that capture alone: an eager call, or another capture,
+    computes its own (an abandoned capture can therefore never hand anyone an unwritten buffer)."""
     if not BALANCED_ORDER or n < 2 or n > 4096 or splits > 1:
         return None
     key = (lens.data_ptr(), n, num_kv_heads)
-    cached = getattr(infer_state, "_morphkv_decode_order", None)
     stream = torch.cuda.current_stream()
-    capturing = torch.cuda.is_current_stream_capturing()
-    if cached is None or cached[0] != key:
+    capture = _capi.capture_id(stream.cuda_stream)          # None outside a capture
+    cached = getattr(infer_state, "_morphkv_decode_order", None)
+    if cached is None or cached[0] != key or cached[4] != capture:
         order = torch.empty(n, dtype=torch.int32, device=lens.device)
-        cached = [key, order, None, stream.cuda_stream]
+        cached = [key, order, None, stream.cuda_stream, capture]
         try:
             infer_state._morphkv_decode_order = cached
         except AttributeError:          # nowhere to keep it: a launch per layer would cost more than it brings
             return None
         _capi.check(_capi.lib().mkv_decode_order(lens.data_ptr(), n, num_kv_heads, order.data_ptr(),
                                                  stream.cuda_stream))
-        if not capturing:
+        if capture is None:
             cached[2] = torch.cuda.Event()
             cached[2].record(stream)
-    elif cached[3] != stream.cuda_stream and cached[2] is not None and not capturing:
+    elif cached[3] != stream.cuda_stream and cached[2] is not None and capture is None:
         stream.wait_event(cached[2])    # computed on another stream
     return cached[1]
 

@@ -6,7 +6,6 @@
 #include <string.h>
 
 #include "morphkv.h"
-#include "morphkv_diag.h"
 
 #define CHECK(cond)                                                          \
     do {                                                                     \
@@ -42,7 +41,7 @@ int main(void) {
 
     /* argument validation comes before any launch */
     CHECK(mkv_append_decode(NULL, NULL, NULL, NULL, 0, NULL, NULL, 1, 0, NULL) == MKV_EINVAL);
-    CHECK(mkv_prof_collect(MKV_K_COUNT, NULL, NULL) == MKV_EINVAL);
+    CHECK(mkv_fill_zero(NULL, 64, NULL) == MKV_EINVAL);
 
     printf("abi_consumer: ok (version %d, sizeof(mkv_pool) %d)\n", mkv_version(), mkv_sizeof_pool());
     return 0;

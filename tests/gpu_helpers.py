@@ -1,12 +1,34 @@
 """Moves seeded scenarios onto the GPU and reads the state back for bit-exact comparison."""
 from __future__ import annotations
 
+import contextlib
+
 import numpy as np
 import torch
 
 from oracle import ref_cpu as R
 from helpers import Case, Cfg
-from morphserve_amd import BlockManager, ElasticKVPool, build_infer_state
+from morphserve_amd import BlockManager, ElasticKVPool, _capi, build_infer_state
+
+
+@contextlib.contextmanager
+def kernel_variant(decode: int = 0, prefill: int = 0):
+    """Pin a kernel variant for the block.  0 / 0 is the product library's own choice and runs on the
+    product library.  Anything else routes the package through the diagnostic twin for the block: it is
+    built from the same sources and also holds the kernels the product never launches (the vector-ALU
+    decode kernel for groups of 4 and 8, the matrix-core one for 1 and 2) and the switches that force a
+    decode kernel (1 vector ALU, 2 matrix cores) or a prefill workgroup shape (4 / 8 waves, pairing bits)."""
+    if not decode and not prefill:
+        yield _capi.lib()
+        return
+    with _capi.use_diag_library() as lib:
+        _capi.check(lib.mkv_set_decode_variant(decode))
+        _capi.check(lib.mkv_set_prefill_variant(prefill))
+        try:
+            yield lib
+        finally:
+            lib.mkv_set_decode_variant(0)
+            lib.mkv_set_prefill_variant(0)
 
 
 def to_gpu(case: Case, dev):

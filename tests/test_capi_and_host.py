@@ -11,8 +11,8 @@ from oracle import ref_cpu as R
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADERS = [os.path.join(ROOT, "include", "morphkv.h"), os.path.join(ROOT, "include", "morphkv_diag.h")]
-DIAG_ONLY = ("mkv_set_decode_variant", "mkv_set_prefill_variant", "mkv_diag_mfma_loop", "mkv_prof_enable",
-             "mkv_prof_reset", "mkv_prof_collect")
+DIAG_ONLY = ("mkv_set_decode_variant", "mkv_set_prefill_variant", "mkv_diag_mfma_loop", "mkv_diag_timeline",
+             "mkv_diag_slab_gather", "mkv_prof_enable", "mkv_prof_reset", "mkv_prof_collect")
 
 
 def _declared(headers=HEADERS):
@@ -40,13 +40,29 @@ def test_header_declares_the_expected_surface():
         assert must in names
 
 
-def test_library_exports_every_declared_symbol():
+def _exported(path):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+
+
+def test_library_exports_exactly_the_declared_symbols():
+    """The product library exports what morphkv.h declares and nothing else (no diagnostics, no C++
+    helpers); its diagnostic twin adds exactly what morphkv_diag.h declares."""
     from morphserve_amd import _capi
     lib = _capi.lib()
-    for name in _declared():
+    boundary = _declared(HEADERS[:1])
+    for name in boundary:
         assert hasattr(lib, name), f"{name} is declared in morphkv.h but not exported"
         assert name in _capi.PROTOTYPES, f"{name} has no ctypes prototype"
-    assert lib.mkv_version() >= 1
+    assert sorted(_capi.PROTOTYPES) == boundary
+    assert _exported(_capi.LIB_PATH) == boundary
+    for name in DIAG_ONLY:
+        assert not hasattr(lib, name), f"{name} is a diagnostic and must not be in the product library"
+    diag = _capi.diag_lib()
+    assert sorted(_capi.DIAG_PROTOTYPES) == sorted(DIAG_ONLY) == _declared(HEADERS[1:])
+    assert _exported(_capi.DIAG_LIB_PATH) == _declared()
+    assert lib.mkv_version() >= 1 and diag.mkv_version() == lib.mkv_version()
     assert ctypes.sizeof(_capi.MkvPool) == lib.mkv_sizeof_pool() == 56 + 2 * 8 * _capi.MKV_MAX_SEGMENTS
 
 
@@ -187,6 +203,8 @@ def test_bad_arguments_are_refused_before_any_launch():
         "mkv_arena_create": (0, 0, None),
         "mkv_arena_resize": (None, 0),
         "mkv_arena_move_tail": (None, None, 4096),
+    }
+    diag_calls = {
         "mkv_diag_slab_gather/not a power of two": (A, A, 1000, 8, 8, 4, 2, 0, 0, A, None),
         "mkv_diag_slab_gather/loads in flight": (A, A, 1024, 8, 8, 3, 2, 0, 0, A, None),
         "mkv_diag_slab_gather/unaligned": (A + 64, A, 1024, 8, 8, 4, 2, 0, 0, A, None),
@@ -196,11 +214,13 @@ def test_bad_arguments_are_refused_before_any_launch():
         "mkv_diag_mfma_loop": (7, 1, None, None, None, None),
         "mkv_prof_collect": (_capi.K_ROPE_STORE + 1, None, None),
     }
-    for name, args in calls.items():
-        fn = getattr(lib, name.split("/")[0])
-        rc = fn(*args)
-        assert rc < 0, f"{name} accepted bad arguments (returned {rc})"
-        assert lib.mkv_last_error(), f"{name} failed without a message"
+    diag = _capi.diag_lib()
+    for handle, table in ((lib, calls), (diag, calls), (diag, diag_calls)):      # the twin refuses the same calls
+        for name, args in table.items():
+            fn = getattr(handle, name.split("/")[0])
+            rc = fn(*args)
+            assert rc < 0, f"{name} accepted bad arguments (returned {rc})"
+            assert handle.mkv_last_error(), f"{name} failed without a message"
 
 
 def test_model_config_kv_sizes_known_answers(tmp_path):

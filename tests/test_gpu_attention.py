@@ -10,7 +10,7 @@ import torch
 
 from oracle import ref_cpu as R
 from helpers import Cfg, assert_attn_close, make_case, rand_f16
-from gpu_helpers import bits, configs, to_gpu
+from gpu_helpers import bits, configs, kernel_variant, to_gpu
 from morphserve_amd import _capi, build_infer_state, paged_attention, store_kvcache
 from morphserve_amd.worker.kernels import paged_attn as PA
 
@@ -27,16 +27,15 @@ def _attend(case, dev, q, layer, policy="auto", target_wgs=None, k_new=(), v_new
     # o arrives 2-D [n, Hq*D] in the reference's layer (a row slice of the hidden state)
     o = torch.full((n, case.Hq * case.D), float("nan"), dtype=torch.float16, device=dev)
     old = (PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS)
-    _capi.check(_capi.lib().mkv_set_decode_variant(variant))   # 0 auto, 1 vector ALU, 2 matrix cores
     PA.SPLIT_POLICY = policy
     if target_wgs is not None:
         PA.TARGET_WORKGROUPS = target_wgs
     try:
-        paged_attention(torch.from_numpy(q).to(dev), kc, vc, list(k_new), list(v_new), bt, model,
-                        engine, st, layer, o)
+        with kernel_variant(decode=variant):                    # 0 auto, 1 vector ALU, 2 matrix cores
+            paged_attention(torch.from_numpy(q).to(dev), kc, vc, list(k_new), list(v_new), bt, model,
+                            engine, st, layer, o)
     finally:
         PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS = old
-        _capi.lib().mkv_set_decode_variant(0)
     torch.cuda.synchronize()
     return o.cpu().numpy().reshape(n, case.Hq, case.D)
 
@@ -209,13 +208,12 @@ def test_fused_append_and_attend(cuda, Hq, Hkv, variant, target_wgs):
     o = torch.full((n, Hq * case.D), float("nan"), dtype=torch.float16, device=cuda)
     old = PA.TARGET_WORKGROUPS
     PA.TARGET_WORKGROUPS = target_wgs
-    _capi.check(_capi.lib().mkv_set_decode_variant(variant))
     try:
-        decode_append_and_attend(torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda),
-                                 torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, 1, o)
+        with kernel_variant(decode=variant):
+            decode_append_and_attend(torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda),
+                                     torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, 1, o)
     finally:
         PA.TARGET_WORKGROUPS = old
-        _capi.lib().mkv_set_decode_variant(0)
     torch.cuda.synchronize()
     assert np.array_equal(bits(kc), bits(case.k_pool)), "K cache after the fused append"
     assert np.array_equal(bits(vc), bits(case.v_pool)), "V cache after the fused append"

@@ -12,7 +12,7 @@ import torch
 
 from oracle import ref_cpu as R
 from helpers import Cfg, assert_attn_close, make_case, rand_f16
-from gpu_helpers import bits, configs, to_gpu
+from gpu_helpers import bits, configs, kernel_variant, to_gpu
 from morphserve_amd import (_capi, build_infer_state, chunked_prefill_attention, decode_append_and_attend,
                             paged_attention, prefill_attention, store_kvcache)
 from morphserve_amd.worker.kernels import paged_attn as PA
@@ -50,15 +50,14 @@ def test_random_decode_attention(cuda, seed):
     o = torch.full((n, Hq * 128), float("nan"), dtype=torch.float16, device=cuda)
     old = (PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS)
     G = Hq // Hkv
-    variant = int(rng.choice([1, 2])) if G in (1, 2, 4, 8) else 0
-    _capi.check(_capi.lib().mkv_set_decode_variant(variant))
+    variant = int(rng.choice([0, 1, 2])) if G in (1, 2, 4, 8) else 0      # 0: the product library and its choice
     PA.SPLIT_POLICY = str(rng.choice(["auto", "reference"]))
     PA.TARGET_WORKGROUPS = int(rng.choice([1, 64, 512, 100000]))
     try:
-        paged_attention(torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, layer, o)
+        with kernel_variant(decode=variant):
+            paged_attention(torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, layer, o)
     finally:
         PA.SPLIT_POLICY, PA.TARGET_WORKGROUPS = old
-        _capi.lib().mkv_set_decode_variant(0)
     torch.cuda.synchronize()
     want = R.paged_attention(q, case.arena, case.lay, case.block_table, case.seq_ids, case.seq_lens, 128 ** -0.5, layer)
     assert_attn_close(o.cpu().numpy().reshape(n, Hq, 128), want,
@@ -106,11 +105,8 @@ def test_random_prefill_and_chunked_prefill(cuda, seed):
     # workgroup shape and tile pairing: the library's choice, or pinned (small grids never pick the paired and the
     # 256-row shapes by themselves): bits 0-7 waves, bits 8-9 pairing forced on (1) / off (2)
     variant = int(rng.choice([0, 4 | (1 << 8), 4 | (2 << 8), 8 | (1 << 8), 8 | (2 << 8)]))
-    _capi.check(_capi.lib().mkv_set_prefill_variant(variant))
-    try:
+    with kernel_variant(prefill=variant):
         _random_prefill_case(cuda, seed, rng, Hq, Hkv, n, lens, variant)
-    finally:
-        _capi.check(_capi.lib().mkv_set_prefill_variant(0))
 
 
 def _random_prefill_case(cuda, seed, rng, Hq, Hkv, n, lens, variant):

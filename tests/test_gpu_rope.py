@@ -7,7 +7,7 @@ import torch
 from oracle import ref_cpu as R
 from oracle import rope_cpu as RO
 from helpers import make_case, rand_f16
-from gpu_helpers import bits, configs, to_gpu
+from gpu_helpers import bits, configs, kernel_variant, to_gpu
 from morphserve_amd import (build_infer_state, rotary_embedding_and_store_kvcache, rotary_embedding_inplace,
                             rotary_tables, store_kvcache)
 
@@ -111,13 +111,12 @@ def test_decode_with_rotary_append_and_attention_in_one_launch(cuda, Hq, Hkv, va
     o = torch.full((n, Hq * case.D), float("nan"), dtype=torch.float16, device=cuda)
     old = PA.TARGET_WORKGROUPS
     PA.TARGET_WORKGROUPS = target_wgs
-    _capi.check(_capi.lib().mkv_set_decode_variant(variant))
     try:
-        decode_rope_append_and_attend(kg, vg, qg, kc, vc, [], [], bt, model, engine, state, layer, o)
-        torch.cuda.synchronize()
+        with kernel_variant(decode=variant):
+            decode_rope_append_and_attend(kg, vg, qg, kc, vc, [], [], bt, model, engine, state, layer, o)
+            torch.cuda.synchronize()
     finally:
         PA.TARGET_WORKGROUPS = old
-        _capi.lib().mkv_set_decode_variant(0)
     assert np.array_equal(bits(qg), bits(q)) and np.array_equal(bits(kg), bits(k))      # inputs untouched
     q_rot, k_rot = q.copy(), k.copy()
     RO.rotary_embedding_inplace(q_rot, k_rot, cos, sin)

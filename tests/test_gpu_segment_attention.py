@@ -14,7 +14,7 @@ import torch
 from oracle import ref_cpu as R
 from oracle import rope_cpu as RO
 from helpers import Cfg, assert_attn_close, rand_f16
-from gpu_helpers import bits
+from gpu_helpers import bits, kernel_variant
 from morphserve_amd import (_capi, build_infer_state, chunked_prefill_attention, decode_append_and_attend,
                             decode_rope_append_and_attend, paged_attention, store_kvcache)
 from morphserve_amd.worker.kernels import paged_attn as PA
@@ -79,11 +79,12 @@ class _Knobs:
     def __enter__(self):
         self.old = PA.TARGET_WORKGROUPS
         PA.TARGET_WORKGROUPS = self.target_wgs
-        _capi.check(_capi.lib().mkv_set_decode_variant(self.variant))
+        self.pin = kernel_variant(decode=self.variant)
+        self.pin.__enter__()
 
     def __exit__(self, *exc):
         PA.TARGET_WORKGROUPS = self.old
-        _capi.lib().mkv_set_decode_variant(0)
+        self.pin.__exit__(*exc)
 
 
 @pytest.mark.parametrize("Hq,Hkv,variant", [(8, 8, 1), (32, 8, 1), (32, 8, 2), (16, 2, 2), (6, 2, 2)])
@@ -182,7 +183,6 @@ def test_attention_through_the_strided_convention(cuda, Hq, Hkv, variant, tps):
     """The reference's calling convention reaches the attention kernels through the C-ABI: only segment 0 is
     passed and mkv_pool_set_strided derives the rest (csrc/src/block_swapping.cpp:156-160)."""
     c = SegCase(cuda, 120 + Hq, Hq, Hkv)
-    lib = _capi.lib()
     pool = pool_strided(c.kc, c.vc, c.k_new[0], c.v_new[0], ORG, c.stride, S, 2, NSEG)
     assert [pool.k_seg[j] for j in range(NSEG)] == [t.data_ptr() for t in c.k_new]
     rng = np.random.default_rng(Hq + 4)
@@ -196,8 +196,7 @@ def test_attention_through_the_strided_convention(cuda, Hq, Hkv, variant, tps):
     mid_o = torch.empty(rows * 128, dtype=torch.float32, device=cuda)
     mid_lse = torch.empty(rows, dtype=torch.float32, device=cuda)
     o = torch.full((n, Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
-    _capi.check(lib.mkv_set_decode_variant(variant))
-    try:
+    with kernel_variant(decode=variant) as lib:
         _capi.check(lib.mkv_paged_attn_decode(
             qg.data_ptr(), o.data_ptr(), C.byref(pool), c.bt.data_ptr(), MBPS, ids.data_ptr(), lens.data_ptr(), n, Hq,
             float(128 ** -0.5), LAYER, tps, splits, mid_o.data_ptr(), mid_lse.data_ptr(), _capi.current_stream()))
@@ -210,8 +209,6 @@ def test_attention_through_the_strided_convention(cuda, Hq, Hkv, variant, tps):
             o.data_ptr(), C.byref(pool), c.bt.data_ptr(), MBPS, ids.data_ptr(), lens.data_ptr(), n, Hq,
             float(128 ** -0.5), LAYER, tps, splits, mid_o.data_ptr(), mid_lse.data_ptr(), _capi.current_stream()))
         torch.cuda.synchronize()
-    finally:
-        lib.mkv_set_decode_variant(0)
     assert np.array_equal(bits(c.g), bits(c.arena)), "whole arena after the fused append (strided pool)"
     assert_attn_close(o.cpu().numpy(), c.oracle(q), f"fused append, strided pool, {splits} splits")
 

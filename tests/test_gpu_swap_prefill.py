@@ -5,7 +5,7 @@ import torch
 
 from oracle import ref_cpu as R
 from helpers import Cfg, assert_attn_close, make_case, rand_f16
-from gpu_helpers import bits, configs, to_gpu
+from gpu_helpers import bits, configs, kernel_variant, to_gpu
 from morphserve_amd import (_capi, build_infer_state, chunked_prefill_attention, prefill_attention,
                             store_kvcache, swiftllm_c)
 from test_gpu_append import _segment_setup
@@ -134,8 +134,7 @@ def test_prefill_attention_both_workgroup_shapes(cuda, waves):
     kc, vc, bt = to_gpu(case, cuda)
     model, engine = configs(case)
     st = build_infer_state(lens.tolist(), case.seq_ids.tolist(), [], Hkv, 128)
-    _capi.check(_capi.lib().mkv_set_prefill_variant(waves))
-    try:
+    with kernel_variant(prefill=waves):
         o = torch.full((T, Hq, 128), float("nan"), dtype=torch.float16, device=cuda)
         prefill_attention(torch.from_numpy(q).to(cuda), torch.from_numpy(k).to(cuda), torch.from_numpy(v).to(cuda),
                           o, model, engine, st)
@@ -151,8 +150,6 @@ def test_prefill_attention_both_workgroup_shapes(cuda, waves):
         chunked_prefill_attention(torch.from_numpy(q2).to(cuda), kc, vc, [], [], bt, model, engine, st2, 0, o2,
                                   prefix_lens=torch.from_numpy(prefix.astype(np.int32)).to(cuda))
         torch.cuda.synchronize()
-    finally:
-        _capi.check(_capi.lib().mkv_set_prefill_variant(0))
     want2 = np.concatenate([want[starts[b] + prefix[b]:starts[b] + lens[b]] for b in range(len(lens))])
     assert_attn_close(o2.cpu().numpy(), want2, f"chunk over prefix, {waves} waves")
 

@@ -1,6 +1,10 @@
 """The per-workgroup time stamps (``mkv_diag_timeline``): a measurement hook that must not change a result.
 
-With a buffer set, the prefill kernel and both decode phase-1 kernels stamp the GPU's constant-rate counter at
+The hook lives in the diagnostic twin of the library only (``libmorphkv_diag.so``); the product library's
+kernels carry no time-stamp argument.  The reference results below come from the PRODUCT library, the
+stamped ones from the twin, so the test also pins that the two libraries compute the same bits.
+
+With a buffer set, the twin's prefill kernel and both decode phase-1 kernels stamp the GPU's constant-rate counter at
 fixed points of every workgroup's life; outputs must be the same bits as without it, the stamps of a workgroup
 must be in order, and with the buffer taken away nothing may be written.
 """
@@ -9,7 +13,7 @@ import pytest
 import torch
 
 from helpers import make_case, rand_f16
-from gpu_helpers import bits, configs, to_gpu
+from gpu_helpers import bits, configs, kernel_variant, to_gpu
 from morphserve_amd import _capi, build_infer_state, paged_attention, prefill_attention
 from morphserve_amd.worker.kernels import paged_attn as PA
 
@@ -18,13 +22,15 @@ POINTS = 8
 
 
 def _stamped(cuda, fn, max_wgs):
+    """``fn`` through the diagnostic twin while it holds a time-stamp buffer for ``max_wgs`` workgroups."""
     buf = torch.zeros(max_wgs * POINTS, dtype=torch.int64, device=cuda)
-    _capi.check(_capi.lib().mkv_diag_timeline(buf.data_ptr(), max_wgs))
-    try:
-        out = fn()
-        torch.cuda.synchronize()
-    finally:
-        _capi.check(_capi.lib().mkv_diag_timeline(None, 0))
+    with _capi.use_diag_library() as lib:
+        _capi.check(lib.mkv_diag_timeline(buf.data_ptr(), max_wgs))
+        try:
+            out = fn()
+            torch.cuda.synchronize()
+        finally:
+            _capi.check(lib.mkv_diag_timeline(None, 0))
     return out, buf.cpu().numpy().reshape(max_wgs, POINTS)
 
 
@@ -54,12 +60,9 @@ def test_prefill_stamps_leave_the_output_alone(cuda):
     plain = run()
     torch.cuda.synchronize()
     for variant in (4 | (1 << 8), 4 | (2 << 8), 8 | (1 << 8)):      # two tiles per workgroup, one, the 256-row shape
-        _capi.check(_capi.lib().mkv_set_prefill_variant(variant))
-        try:
+        with kernel_variant(prefill=variant):
             ref = run()
             got, stamps = _stamped(cuda, run, 4096)
-        finally:
-            _capi.check(_capi.lib().mkv_set_prefill_variant(0))
         assert np.array_equal(bits(got), bits(ref)) and np.array_equal(bits(got), bits(plain))
         live = _in_order(stamps)
         ran = live[live[:, 1] > 0]                                  # slots past a short sequence's tiles leave at once
