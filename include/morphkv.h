@@ -324,6 +324,36 @@ int mkv_arena_destroy(mkv_arena* arena);
  * chunk in hand returns to `from`, chunks already moved stay in `to`
  * (mkv_arena_info tells how far it got). */
 int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes);
+/* Pool creation and growth that choose WHICH physical memory backs K and which backs V.  The
+ * reference allocates k_cache and v_cache one after the other (MS/worker/model.py:187-190) and
+ * carves K and V of a new segment out of one range (CS/memory_manager.cpp:120-145), so where they
+ * lie is the driver's choice.  On an MI355X that choice matters: its memory behaves as three groups
+ * of 96 GiB, the migration copy of a shrink runs at 65 % of the HBM peak when the K and the V
+ * destinations share a group and at 78 % when they do not, and the decode gather is fastest over a
+ * pool that touches at most two groups.  mkv_arena_pair_grow maps k_add_bytes more at the end of
+ * `k` and v_add_bytes more at the end of `v` (both arenas of one pool: same chunk size and device)
+ * with K chunks from one group and V chunks from another: it creates candidate chunks (at most
+ * budget_bytes of them at a time, 0 = all free device memory but 4 GiB), tells their groups apart by
+ * the rate of a store-only kernel that fills a candidate and a reference side by side (a relative
+ * measurement: no absolute rate is assumed, and a device without such groups yields one group and
+ * the plain order), keeps what it needs, preferring each arena's own group, and gives the rest back.
+ * Where an arena can still grow it also keeps one spare chunk of its group as the reference for the
+ * next call (held until mkv_arena_destroy).  Chunks under 256 MiB cannot be measured: plain growth.
+ * Host call; it synchronises `stream`, on which the measurement kernels run; the new memory holds
+ * whatever the measurement left (the caller clears it, as after mkv_arena_resize).  MKV_ENOSPC when
+ * the device has no memory left (nothing changed).  `info` (may be NULL) reports what was found. */
+typedef struct mkv_pair_info {
+    int32_t groups_found;   /* 0: not measured (plain growth), 1: one group only, 2 or 3 */
+    int32_t candidates;     /* physical chunks created by the call */
+    int32_t k_chunks, v_chunks;         /* chunks mapped into k / v */
+    int32_t k_in_group, v_in_group;     /* ... of which in the arena's own group */
+    int32_t probes;         /* measurement launches (x 3) */
+    int32_t _pad;
+    double probe_ms;        /* GPU time of the measurement */
+    double total_ms;        /* host time of the call */
+} mkv_pair_info;
+int mkv_arena_pair_grow(mkv_arena* k, mkv_arena* v, uint64_t k_add_bytes, uint64_t v_add_bytes,
+                        uint64_t budget_bytes, void* stream, mkv_pair_info* info);
 
 /* ---- rotary embedding, optionally fused with the append --------------------- */
 /* rotary_embedding_inplace, MS/worker/kernels/rotary_emb.py:7-58: q [T, Hq, D] and

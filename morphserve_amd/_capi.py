@@ -43,6 +43,22 @@ class MkvPool(C.Structure):
     ]
 
 
+class MkvPairInfo(C.Structure):
+    """``mkv_pair_info``: what a memory-group aware growth found (include/morphkv.h)."""
+    _fields_ = [
+        ("groups_found", C.c_int32),
+        ("candidates", C.c_int32),
+        ("k_chunks", C.c_int32),
+        ("v_chunks", C.c_int32),
+        ("k_in_group", C.c_int32),
+        ("v_in_group", C.c_int32),
+        ("probes", C.c_int32),
+        ("_pad", C.c_int32),
+        ("probe_ms", C.c_double),
+        ("total_ms", C.c_double),
+    ]
+
+
 _P = C.c_void_p
 _I32 = C.c_int32
 _I64 = C.c_int64
@@ -86,6 +102,7 @@ PROTOTYPES = {
     "mkv_arena_resize": [_P, _U64],
     "mkv_arena_destroy": [_P],
     "mkv_arena_move_tail": [_P, _P, _U64],
+    "mkv_arena_pair_grow": [_P, _P, _U64, _U64, _U64, _P, C.POINTER(MkvPairInfo)],
     "mkv_rope_store_kvcache": [_P, _P, _P, _P, _P, _PP, _P, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32,
                                _I32, _I32, _I32, _P],
     "mkv_swap_blocks": [_P, _P, _I64, _I32, _PP, _P, _P, C.POINTER(_I64), _P],

@@ -10,29 +10,31 @@ namespace mkv {
 
 static constexpr int kScanThreads = 1024;
 static constexpr int kScanWaves = kScanThreads / 64;
-static constexpr int kBytesPerThread = 16;
-static constexpr int64_t kTileBytes = (int64_t)kScanThreads * kBytesPerThread;
+static constexpr int kBytesPerThread = 64;                 // four 16-byte loads in flight per thread
+static constexpr int64_t kTileBytes = (int64_t)kScanThreads * kBytesPerThread;      // 64 Ki map bytes per round
+static constexpr int kIdCache = 4096;                      // ids kept in LDS between the taking and the handing out
 
 // Exclusive prefix sum over the workgroup (1024 threads); total returned in *total.
 // All threads must call it.
-__device__ __forceinline__ int64_t block_excl_scan(int64_t v, int64_t* total, int64_t* sm /* [kScanWaves + 1] */) {
+template <typename T>
+__device__ __forceinline__ T block_excl_scan(T v, T* total, T* sm /* [kScanWaves + 1] */) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    int64_t inc = v;
+    T inc = v;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
-        int64_t t = __shfl_up(inc, d);
+        T t = __shfl_up(inc, d);
         if (lane >= d) inc += t;
     }
     __syncthreads();                       // sm reuse across calls
     if (lane == 63) sm[wave] = inc;
     __syncthreads();
     if (wave == 0) {
-        int64_t w = lane < kScanWaves ? sm[lane] : 0;
-        int64_t winc = w;
+        T w = lane < kScanWaves ? sm[lane] : 0;
+        T winc = w;
 #pragma unroll
         for (int d = 1; d < kScanWaves; d <<= 1) {
-            int64_t t = __shfl_up(winc, d);
+            T t = __shfl_up(winc, d);
             if (lane >= d) winc += t;
         }
         if (lane < kScanWaves) sm[lane] = winc - w;       // exclusive wave offsets
@@ -43,33 +45,41 @@ __device__ __forceinline__ int64_t block_excl_scan(int64_t v, int64_t* total, in
     return sm[wave] + inc - v;
 }
 
-// One thread's 16 map bytes starting at b0 (16-byte aligned as an address) as a bit mask: bit k is
-// set when byte b0 + k lies in [lo, hi) and is non-zero (want != 0) or zero (want == 0).  A unit
-// that lies wholly inside the range is one 16-byte load.
-__device__ __forceinline__ uint32_t match_mask16(const uint8_t* map, int64_t b0, int64_t lo, int64_t hi,
-                                                uint8_t want) {
-    if (b0 + kBytesPerThread <= lo || b0 >= hi) return 0u;
-    uint32_t nz = 0u, in = 0xffffu;
+// 16 map bytes as a 16-bit mask of the non-zero ones.
+__device__ __forceinline__ uint32_t nonzero_mask16(const uint4 w) {
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+    uint32_t nz = 0u;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t t = words[q];
+        t |= t >> 4;
+        t |= t >> 2;
+        t |= t >> 1;
+        t &= 0x01010101u;                                   // one flag per non-zero byte
+        nz |= (((t * 0x01020408u) >> 24) & 0xfu) << (4 * q);
+    }
+    return nz;
+}
+
+// One thread's 64 map bytes starting at b0 (16-byte aligned as an address) as a bit mask: bit k is
+// set when byte b0 + k lies in [lo, hi) and is non-zero (want != 0) or zero (want == 0).  A thread
+// whose bytes lie wholly inside the range issues four independent 16-byte loads.
+__device__ __forceinline__ uint64_t match_mask64(const uint8_t* map, int64_t b0, int64_t lo, int64_t hi,
+                                                 uint8_t want) {
+    if (b0 + kBytesPerThread <= lo || b0 >= hi) return 0ull;
+    uint64_t nz = 0ull, in = ~0ull;
     if (b0 >= lo && b0 + kBytesPerThread <= hi) {
-        const uint4 w = *(const uint4*)(map + b0);
-        const uint32_t words[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            uint32_t t = words[q];
-            t |= t >> 4;
-            t |= t >> 2;
-            t |= t >> 1;
-            t &= 0x01010101u;                                   // one flag per non-zero byte
-            nz |= (((t * 0x01020408u) >> 24) & 0xfu) << (4 * q);
-        }
+        const uint4* p = (const uint4*)(map + b0);
+        const uint4 w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3];
+        nz = (uint64_t)nonzero_mask16(w0) | ((uint64_t)nonzero_mask16(w1) << 16) |
+             ((uint64_t)nonzero_mask16(w2) << 32) | ((uint64_t)nonzero_mask16(w3) << 48);
     } else {
-        in = 0u;
-#pragma unroll
+        in = 0ull;
         for (int k = 0; k < kBytesPerThread; ++k) {
             const int64_t b = b0 + k;
             if (b >= lo && b < hi) {
-                in |= 1u << k;
-                if (map[b] != 0) nz |= 1u << k;
+                in |= 1ull << k;
+                if (map[b] != 0) nz |= 1ull << k;
             }
         }
     }
@@ -77,7 +87,7 @@ __device__ __forceinline__ uint32_t match_mask16(const uint8_t* map, int64_t b0,
 }
 
 // The scans below walk [lo, hi) in tiles of kTileBytes that start at an address multiple of 16, so
-// that every thread's unit can be one aligned 16-byte load whatever lo and the map's own alignment.
+// that every thread's bytes can be aligned 16-byte loads whatever lo and the map's own alignment.
 __device__ __forceinline__ int64_t aligned_start(const uint8_t* map, int64_t lo) {
     return lo - (int64_t)(((uintptr_t)map + (uint64_t)lo) & 15u);
 }
@@ -85,45 +95,50 @@ __device__ __forceinline__ int64_t aligned_start(const uint8_t* map, int64_t lo)
 // Counts bytes equal to `want` in map[lo, hi) until at least `limit` are seen
 // (early exit at tile granularity).  All threads must call it.
 __device__ int64_t count_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8_t want,
-                               int64_t limit, int64_t* sm) {
+                               int64_t limit, int32_t* sm) {
     int64_t seen = 0;
     for (int64_t t0 = aligned_start(map, lo); t0 < hi && seen < limit; t0 += kTileBytes) {
         const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
-        const int64_t c = __popc(match_mask16(map, b0, lo, hi, want));
-        int64_t tot;
-        block_excl_scan(c, &tot, sm);
+        const int32_t c = __popcll(match_mask64(map, b0, lo, hi, want));
+        int32_t tot;
+        block_excl_scan<int32_t>(c, &tot, sm);
         seen += tot;
     }
     return seen;
 }
 
-// Writes the first `n` positions of map[lo, hi) whose byte equals `want` (in
-// ascending order) to out[0..n) and stores `mark` there.  The caller has
-// verified that at least n exist.  All threads must call it.
-__device__ void take_bytes(uint8_t* map, int64_t lo, int64_t hi, uint8_t want, uint8_t mark,
-                           int64_t n, int64_t* out, int64_t* sm) {
+// Writes the first `n` positions of map[lo, hi) whose byte equals `want`, ascending, to out[0..n)
+// (and the first kIdCache of them to `cache`, when given) WITHOUT touching the map; returns how many
+// were found, which is below n only when the range holds fewer.  `first_bits` / `have_first`: the
+// mask of the first tile when the caller has requested it early.  All threads must call it.
+__device__ int64_t collect_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8_t want, int64_t n,
+                                 int64_t* out, int32_t* cache, int32_t* sm, uint64_t first_bits, bool have_first) {
     int64_t base = 0;
+    bool first = true;
     for (int64_t t0 = aligned_start(map, lo); t0 < hi && base < n; t0 += kTileBytes) {
         const int64_t b0 = t0 + (int64_t)threadIdx.x * kBytesPerThread;
-        const uint32_t bits = match_mask16(map, b0, lo, hi, want);
-        const int64_t c = __popc(bits);
-        int64_t tot;
-        int64_t pos = base + block_excl_scan(c, &tot, sm);
-#pragma unroll
-        for (int k = 0; k < kBytesPerThread; ++k) {
-            if ((bits >> k) & 1u) {
-                if (pos < n) {
-                    out[pos] = b0 + k;
-                    map[b0 + k] = mark;
-                }
-                ++pos;
-            }
+        uint64_t bits = (first && have_first) ? first_bits : match_mask64(map, b0, lo, hi, want);
+        first = false;
+        const int32_t c = __popcll(bits);
+        int32_t tot;
+        int64_t pos = base + block_excl_scan<int32_t>(c, &tot, sm);
+        while (bits != 0ull && pos < n) {
+            const int k = __builtin_ctzll(bits);
+            bits &= bits - 1;
+            out[pos] = b0 + k;
+            if (cache != nullptr && pos < kIdCache) cache[pos] = (int32_t)(b0 + k);
+            ++pos;
         }
         base += tot;
     }
+    return base < n ? base : n;
 }
 
 // ---- allocate_blocks_for_seqs, fused ---------------------------------------------
+// One launch: needs -> do they fit -> the lowest free ids -> the table rows.  The first 64 Ki map
+// bytes are requested before anything else, so that their trip to memory overlaps the trip for the
+// rows' counts; ids are collected first and the map is only marked once the request is known to fit,
+// so a refused call changes nothing but the scratch in new_ids.
 __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
     int32_t* __restrict__ n_alloc, int32_t* __restrict__ block_table, int64_t max_blocks_per_seq,
     uint8_t* __restrict__ is_free, int64_t num_blocks, const int32_t* __restrict__ seq_ids,
@@ -131,9 +146,13 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
     int64_t* __restrict__ new_ids, int64_t new_ids_cap, int64_t* __restrict__ result,
     int64_t max_seqs) {
     __shared__ int64_t sm[kScanWaves + 1];
+    __shared__ int32_t s_ids[kIdCache];
     __shared__ int s_bad;
+    int32_t* sm32 = (int32_t*)sm;
     const int tid = threadIdx.x;
     if (tid == 0) s_bad = 0;
+    const uint64_t first_bits = match_mask64(is_free, aligned_start(is_free, 0) + (int64_t)tid * kBytesPerThread, 0,
+                                             num_blocks, 1);
     __syncthreads();
 
     // pass 1: total need, precondition need_i >= 0 and room in the table row
@@ -149,7 +168,7 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
         my_need += need;
     }
     int64_t total;
-    block_excl_scan(my_need, &total, sm);
+    block_excl_scan<int64_t>(my_need, &total, sm);
     __syncthreads();
     if (s_bad) {
         if (tid == 0) { result[0] = total; result[1] = (s_bad == 2) ? MKV_EINVAL : MKV_ELOGIC; result[2] = 0; }
@@ -159,16 +178,21 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
         if (tid == 0) { result[0] = 0; result[1] = MKV_OK; result[2] = 0; }
         return;
     }
-    // pass 2: are there enough free blocks? (no state touched yet)
-    const int64_t found = count_bytes(is_free, 0, num_blocks, 1, total, sm);
-    if (found < total || total > new_ids_cap) {
+    if (total > new_ids_cap) {
+        if (tid == 0) { result[0] = total; result[1] = MKV_ENOSPC; result[2] = 0; }
+        return;
+    }
+    // pass 2: the lowest `total` free ids (the map is not touched yet)
+    const int64_t found = collect_bytes(is_free, 0, num_blocks, 1, total, new_ids, s_ids, sm32, first_bits, true);
+    if (found < total) {
         if (tid == 0) { result[0] = total; result[1] = MKV_ENOSPC; result[2] = found; }
         return;
     }
-    // pass 3: take the lowest `total` free ids
-    take_bytes(is_free, 0, num_blocks, 1, 0, total, new_ids, sm);
     __threadfence_block();
     __syncthreads();
+    // pass 3: they are used from now on
+    for (int64_t p = tid; p < total; p += kScanThreads)
+        is_free[p < kIdCache ? (int64_t)s_ids[p] : new_ids[p]] = 0;
     // pass 4: hand them to the rows in batch order
     int64_t base = 0;
     for (int i0 = 0; i0 < batch; i0 += kScanThreads) {
@@ -180,10 +204,13 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
             need = ((int64_t)target_lens[i] + block_size - 1) / block_size - have;
         }
         int64_t tot;
-        const int64_t start = base + block_excl_scan(need, &tot, sm);
+        const int64_t start = base + block_excl_scan<int64_t>(need, &tot, sm);
         if (i < batch && need > 0) {
             int32_t* dst = block_table + seq * max_blocks_per_seq + have;
-            for (int64_t x = 0; x < need; ++x) dst[x] = (int32_t)new_ids[start + x];
+            for (int64_t x = 0; x < need; ++x) {
+                const int64_t p = start + x;
+                dst[x] = p < kIdCache ? s_ids[p] : (int32_t)new_ids[p];
+            }
             n_alloc[seq] = (int32_t)(have + need);
         }
         base += tot;
@@ -195,12 +222,14 @@ __global__ __launch_bounds__(kScanThreads) void bm_take_first_free_kernel(
     uint8_t* __restrict__ is_free, int64_t num_blocks, int64_t n, int64_t* __restrict__ ids_out,
     int64_t* __restrict__ result) {
     __shared__ int64_t sm[kScanWaves + 1];
-    const int64_t found = count_bytes(is_free, 0, num_blocks, 1, n, sm);
+    const int64_t found = collect_bytes(is_free, 0, num_blocks, 1, n, ids_out, nullptr, (int32_t*)sm, 0ull, false);
     if (found < n) {
         if (threadIdx.x == 0) { result[0] = found; result[1] = MKV_ENOSPC; }
         return;
     }
-    take_bytes(is_free, 0, num_blocks, 1, 0, n, ids_out, sm);
+    __threadfence_block();
+    __syncthreads();
+    for (int64_t p = threadIdx.x; p < n; p += kScanThreads) is_free[ids_out[p]] = 0;
     if (threadIdx.x == 0) { result[0] = n; result[1] = MKV_OK; }
 }
 
@@ -224,7 +253,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_append_kernel(
             if (need < 0) need = 0;
         }
         int64_t tot;
-        const int64_t start = base + block_excl_scan(need, &tot, sm);
+        const int64_t start = base + block_excl_scan<int64_t>(need, &tot, sm);
         if (ok && need > 0) {
             // never write past the row, and never count more entries than the row holds
             const int64_t fit = max((int64_t)0, min(need, max_blocks_per_seq - have));
@@ -263,7 +292,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_release_kernel(
         if (lane == 0 && seq >= 0 && seq < max_seqs) n_alloc[seq] = 0;
     }
     int64_t tot;
-    block_excl_scan(mine, &tot, sm);
+    block_excl_scan<int64_t>(mine, &tot, sm);
     if (threadIdx.x == 0 && freed_total) *freed_total = tot;
 }
 
@@ -282,7 +311,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_gather_release_kernel(
     int64_t mine = 0;
     for (int i = tid; i < batch; i += kScanThreads) mine += count_of(i);
     int64_t total;
-    block_excl_scan(mine, &total, sm);
+    block_excl_scan<int64_t>(mine, &total, sm);
     __syncthreads();
     if (total > capacity) {
         if (tid == 0) { result[0] = total; result[1] = MKV_ENOSPC; }
@@ -295,7 +324,7 @@ __global__ __launch_bounds__(kScanThreads) void bt_gather_release_kernel(
         const int i = i0 + tid;
         const int64_t cnt = (i < batch) ? count_of(i) : 0;
         int64_t tot;
-        const int64_t start = base + block_excl_scan(cnt, &tot, sm);
+        const int64_t start = base + block_excl_scan<int64_t>(cnt, &tot, sm);
         // the thread that owns row i copies it (rows are short: ceil(len/B) entries)
         if (i < batch && cnt > 0) {
             const int64_t seq = seq_ids[i];
@@ -319,30 +348,51 @@ __global__ __launch_bounds__(kScanThreads) void bt_gather_release_kernel(
 __global__ __launch_bounds__(kScanThreads) void bm_count_live_kernel(
     const uint8_t* __restrict__ is_free, int64_t lo, int64_t hi, int64_t* __restrict__ result) {
     __shared__ int64_t sm[kScanWaves + 1];
-    const int64_t live = count_bytes(is_free, lo, hi, 0, INT64_MAX, sm);
+    const int64_t live = count_bytes(is_free, lo, hi, 0, INT64_MAX, (int32_t*)sm);
     if (threadIdx.x == 0) *result = live;
 }
 
 // ---- shrink planning ---------------------------------------------------------------
+// Live ids >= new_n, ascending, move to the lowest free ids < new_n.  Both lists are collected without
+// touching the map; only a plan that fits is applied (sources become free, destinations used, remap
+// holds the new id of every moved block and the identity elsewhere).
 __global__ __launch_bounds__(kScanThreads) void pool_plan_shrink_kernel(
     uint8_t* __restrict__ is_free, int64_t num_blocks, int64_t new_n, int64_t* __restrict__ src,
     int64_t* __restrict__ dst, int64_t cap, int32_t* __restrict__ remap,
     int64_t* __restrict__ result) {
     __shared__ int64_t sm[kScanWaves + 1];
+    int32_t* sm32 = (int32_t*)sm;
     const int tid = threadIdx.x;
-    const int64_t moves = count_bytes(is_free, new_n, num_blocks, 0, INT64_MAX, sm);
-    const int64_t free_below = count_bytes(is_free, 0, new_n, 1, moves, sm);
-    if (free_below < moves || moves > cap) {
-        if (tid == 0) { result[0] = moves; result[1] = MKV_ENOSPC; result[2] = free_below; }
+    // identity first: independent stores that drain while the map is read (four ids per store where the
+    // array's alignment allows)
+    if ((((uintptr_t)remap) & 15u) == 0) {
+        int4* r4 = (int4*)remap;
+        for (int64_t q = tid; q < num_blocks / 4; q += kScanThreads) {
+            const int32_t b = (int32_t)(4 * q);
+            r4[q] = make_int4(b, b + 1, b + 2, b + 3);
+        }
+        for (int64_t b = (num_blocks / 4) * 4 + tid; b < num_blocks; b += kScanThreads) remap[b] = (int32_t)b;
+    } else {
+        for (int64_t b = tid; b < num_blocks; b += kScanThreads) remap[b] = (int32_t)b;
+    }
+    // live blocks above the cut: all of them, as many as the lists hold (one more than `cap` says "too many")
+    const int64_t moves = collect_bytes(is_free, new_n, num_blocks, 0, cap, src, nullptr, sm32, 0ull, false);
+    const int64_t live_above = moves < cap ? moves : count_bytes(is_free, new_n, num_blocks, 0, INT64_MAX, sm32);
+    const int64_t free_below = collect_bytes(is_free, 0, new_n, 1, live_above <= cap ? live_above : 0, dst, nullptr,
+                                             sm32, 0ull, false);
+    if (live_above > cap || free_below < live_above) {
+        const int64_t fb = live_above > cap ? count_bytes(is_free, 0, new_n, 1, live_above, sm32) : free_below;
+        if (tid == 0) { result[0] = live_above; result[1] = MKV_ENOSPC; result[2] = fb; }
         return;
     }
-    for (int64_t b = tid; b < num_blocks; b += kScanThreads) remap[b] = (int32_t)b;
-    // live ids >= new_n ascending become free; lowest free ids < new_n become used
-    take_bytes(is_free, new_n, num_blocks, 0, 1, moves, src, sm);
-    take_bytes(is_free, 0, new_n, 1, 0, moves, dst, sm);
     __threadfence_block();
     __syncthreads();
-    for (int64_t k = tid; k < moves; k += kScanThreads) remap[src[k]] = (int32_t)dst[k];
+    for (int64_t k = tid; k < moves; k += kScanThreads) {
+        const int64_t s_id = src[k], d_id = dst[k];
+        is_free[s_id] = 1;
+        is_free[d_id] = 0;
+        remap[s_id] = (int32_t)d_id;
+    }
     if (tid == 0) { result[0] = moves; result[1] = MKV_OK; result[2] = free_below; }
 }
 

@@ -30,21 +30,24 @@ class ElasticKVPool:
 
     def __init__(self, num_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int,
-                 device: str = "cuda", zero_init: bool = True, tune_placement: Optional[bool] = None,
-                 settle_seconds: Optional[float] = None):
+                 device: str = "cuda", zero_init: bool = True, tune_placement: bool = False,
+                 reserve_blocks: int = 0):
+        """``tune_placement``: let ``kv_placement.allocate_kv_caches`` time a few starting offsets for the V
+        tensor and keep the fastest (off by default).  ``reserve_blocks``: the largest size the pool may grow
+        to, when known (the free map is then allocated once)."""
         _capi.lib()
         self.device = torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
-        # K and V as the reference creates them (model.py:187-190); the V base may sit a few KiB into its
-        # allocation where the decode gather measures faster that way (kv_placement)
+        # K and V as the reference creates them (model.py:187-190); on request the V base may sit a few KiB
+        # into its allocation where the decode gather measures faster that way (kv_placement)
         self.k_cache, self.v_cache, self.kv_placement = allocate_kv_caches(
-            num_blocks, self.shape_tail, device, zero_init=zero_init, tune=tune_placement,
-            settle_seconds=settle_seconds)
+            num_blocks, self.shape_tail, device, zero_init=zero_init, tune=tune_placement)
         self.k_cache_new: List[torch.Tensor] = []
         self.v_cache_new: List[torch.Tensor] = []
         self.kv_cache_new_block_size = 0
         self.block_manager = BlockManager("GPU", num_blocks, max_seqs_in_block_table,
-                                          max_blocks_per_seq, block_size, device=device)
+                                          max_blocks_per_seq, block_size, device=device,
+                                          reserve_blocks=reserve_blocks)
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
 
     # -- description ---------------------------------------------------------------
@@ -91,10 +94,7 @@ class ElasticKVPool:
         bm = self.block_manager
         bm.num_blocks += seg_blocks
         bm.num_free_blocks += seg_blocks
-        new_map = torch.empty(bm.num_blocks, dtype=torch.bool, device=self.device)
-        new_map[:bm.is_block_free.shape[0]] = bm.is_block_free
-        new_map[bm.is_block_free.shape[0]:] = True
-        bm.is_block_free = new_map
+        bm.grow_free_map(seg_blocks)
 
     # -- shrink ------------------------------------------------------------------------
     def tail_segment_unused(self) -> bool:
@@ -122,7 +122,7 @@ class ElasticKVPool:
             del self.v_cache_new[-1]
             bm.num_blocks -= s
             bm.num_free_blocks -= s
-        bm.is_block_free = bm.is_block_free[:bm.num_blocks]
+        bm.shrink_free_map(bm.num_blocks)
         if not self.k_cache_new:
             self.kv_cache_new_block_size = 0
 

@@ -10,15 +10,19 @@ on where the driver placed the allocations, so it is measured, not assumed).
 ``allocate_kv_caches`` allocates V with a few KiB of slack, times the decode gather for a handful of
 V offsets on the freshly allocated memory and returns V as the view that was fastest.  The tensors
 have the reference's shapes and are contiguous; only ``v_cache.data_ptr()`` differs from a plain
-allocation.  ``tune=None`` (the default) does this for pools of ``MIN_BYTES_TO_TUNE`` per tensor and more -- the
-effect was measured on 64-186 GiB pools; on a pool of a few hundred MiB the probe only sees its own noise --
-``tune=True`` for any pool of at least ``MIN_BLOCKS_TO_TUNE`` blocks, ``tune=False`` never (offset 0).
+allocation.  Off by default (``tune=False``: two plain allocations); ``tune=True`` does it for any pool of at
+least ``MIN_BLOCKS_TO_TUNE`` blocks -- the effect was measured on 64-186 GiB pools; on a pool of a few hundred
+MiB the probe only sees its own noise.  The decision is relative (a candidate against offset 0 on the same
+allocation), no rate is assumed.
+
+Which PHYSICAL memory backs the two tensors matters more than this offset and is not something two plain
+allocations can choose: a pool that owns its memory (``vmm_pool.VmmKVPool``) places K and V in different memory
+groups of the device instead (``mkv_arena_pair_grow``).
 """
 from __future__ import annotations
 
 import ctypes as C
-import time
-from typing import Dict, Optional, Sequence, Tuple
+from typing import Dict, Sequence, Tuple
 
 import torch
 
@@ -28,13 +32,6 @@ from . import _capi
 CANDIDATE_OFFSETS = (0, 4096, 8192, 12288, 20480)
 SLACK_BYTES = 32768
 MIN_BLOCKS_TO_TUNE = 4096
-MIN_BYTES_TO_TUNE = 16 << 30
-SETTLE_SECONDS = 12.0
-# The probe on settled / recycled memory, K + V pools of 128 GiB: 6140-6190 / 5650-6035 GB/s; of 186 GiB: 6180-6200 /
-# 5930; of 64 GiB: 6320-6370 / 6000-6090 GB/s (a smaller pool gathers faster).  The line between them:
-SETTLE_BELOW_GBS = 6080.0           # pools of 128 GiB and more
-SETTLE_BELOW_GBS_PER_GIB = -1.9     # added per GiB under 128
-SETTLE_BELOW_MAX = 6250.0
 
 
 def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Sequence[int]) -> float:
@@ -61,44 +58,13 @@ def _probe_us(k_cache: torch.Tensor, v_cache: torch.Tensor, probe, layers: Seque
 
 
 def allocate_kv_caches(num_blocks: int, shape_tail: Tuple[int, int, int, int], device, zero_init: bool = True,
-                       tune: Optional[bool] = None, seed: int = 0,
-                       settle_seconds: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor, Dict]:
-    """``(k_cache, v_cache, info)`` with ``k_cache, v_cache : [num_blocks, L, Hkv, B, D]`` fp16.
-
-    ``settle_seconds`` (``None``: ``SETTLE_SECONDS`` whenever the probe runs, 0: never): for some seconds after
-    a large amount of device memory has been freed -- by this process or by one that has just exited -- the
-    driver hands out memory on which the gather runs 2-7 % slower for as long as the allocation lives; an
-    allocation made ten seconds later is as fast as the first one of a freshly started machine.  When the probe
-    reads less than a threshold calibrated on this GPU (``SETTLE_BELOW_GBS`` for a 128 GiB pool, a little more for a
-    smaller one) the pool is therefore given back, the call sleeps ``settle_seconds`` and
-    allocates and probes once more (never more than once; the second allocation is kept whatever it reads)."""
+                       tune: bool = False, seed: int = 0) -> Tuple[torch.Tensor, torch.Tensor, Dict]:
+    """``(k_cache, v_cache, info)`` with ``k_cache, v_cache : [num_blocks, L, Hkv, B, D]`` fp16."""
     L, hkv, bsz, d = shape_tail
     device = torch.device(device)
-    shape = (num_blocks, L, hkv, bsz, d)
-    numel = num_blocks * L * hkv * bsz * d
     supported = bsz == 16 and d == 128 and device.type == "cuda"
-    if tune is None:
-        tune = numel * 2 >= MIN_BYTES_TO_TUNE
     tune = bool(tune and supported and num_blocks >= MIN_BLOCKS_TO_TUNE)
-    if settle_seconds is None:
-        settle_seconds = SETTLE_SECONDS
-    k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
-    if tune and settle_seconds > 0 and info["probe_GBs"] < _settle_threshold(2 * numel * 2):
-        first = info["probe_GBs"]
-        del k_cache, v_cache
-        torch.cuda.synchronize(device)
-        torch.cuda.empty_cache()
-        time.sleep(settle_seconds)
-        k_cache, v_cache, info = _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
-        info["settled"] = {"first_probe_GBs": first, "waited_s": settle_seconds}
-    return k_cache, v_cache, info
-
-
-def _settle_threshold(pool_bytes: int) -> float:
-    if SETTLE_BELOW_GBS <= 0 or SETTLE_BELOW_GBS >= 1e9:          # switched off / forced (tests)
-        return SETTLE_BELOW_GBS
-    thr = SETTLE_BELOW_GBS + SETTLE_BELOW_GBS_PER_GIB * min(0.0, pool_bytes / 2 ** 30 - 128.0)
-    return min(thr, SETTLE_BELOW_MAX)
+    return _allocate_and_probe(num_blocks, shape_tail, device, zero_init, tune, seed)
 
 
 def _make_probe(num_blocks: int, shape_tail, device, seed: int):
@@ -127,11 +93,6 @@ def probe_gather_GBs(k_cache: torch.Tensor, v_cache: torch.Tensor, seed: int = 0
     probe, layers, probe_bytes = _make_probe(num_blocks, shape_tail, k_cache.device, seed)
     best = min(_probe_us(k_cache, v_cache, probe, layers) for _ in range(3))
     return round(probe_bytes / best / 1e3, 1)
-
-
-def settle_threshold_GBs(pool_bytes: int) -> float:
-    """Below this probe rate a pool of ``pool_bytes`` (K and V together) is taken to lie on recycled memory."""
-    return _settle_threshold(pool_bytes)
 
 
 def _allocate_and_probe(num_blocks: int, shape_tail, device, zero_init: bool, tune: bool, seed: int):

@@ -54,6 +54,9 @@ class PoolEngine:
         self.migrate = migrate
         self.scheduler = None        # set by the owner once the Scheduler exists
         self.migrated_blocks = 0     # live blocks relocated by shrinks so far
+        # blocks each replaced layer gave to the pool: arenas may differ in what they can spare (their size,
+        # the pool's remaining reservation), so a restored layer takes back exactly what IT gave
+        self.blocks_from_layer: Dict[int, int] = {}
 
 
 class _ShrinkInto:
@@ -85,6 +88,7 @@ def update_kvcache_after_replacing_layer(engine: PoolEngine, layer_id: int) -> N
     else:
         model.pool.expand(int(seg[0].shape[0]), seg[0], seg[1])
         model.kv_cache_new_block_size = int(seg[0].shape[0])
+    engine.blocks_from_layer[layer_id] = model.kv_cache_new_block_size
     if engine.scheduler is not None:
         engine.scheduler.num_gpu_blocks += model.kv_cache_new_block_size
 
@@ -119,20 +123,23 @@ def quant2org_and_update_kvcache(engine: PoolEngine, update_kvcache: bool = True
         arena = engine.layer_arenas.get(layer_id)
         if arena is not None:                              # the memory goes back to the layer it came from
             pool = _ShrinkInto(pool, arena)
-        if contiguous and pool.tail_unused(model.kv_cache_new_block_size):
-            pool.shrink_to(pool.num_blocks - model.kv_cache_new_block_size)
+        # what this layer gave (the reference's segments all have one size, so there the latest value does)
+        given = engine.blocks_from_layer.get(layer_id, model.kv_cache_new_block_size)
+        if contiguous and pool.tail_unused(given):
+            pool.shrink_to(pool.num_blocks - given)
         elif not contiguous and pool.shrink_tail_if_unused():
             pass
         elif not engine.migrate:
             return False
         else:
             try:
-                src, _ = pool.shrink_to(pool.num_blocks - model.kv_cache_new_block_size)
+                src, _ = pool.shrink_to(pool.num_blocks - given)
             except PoolTooFullError:       # does not fit: an ordinary refusal; a failed launch propagates
                 return False
             engine.migrated_blocks += int(src.numel())
+        engine.blocks_from_layer.pop(layer_id, None)
         if engine.scheduler is not None:
-            engine.scheduler.num_gpu_blocks -= model.kv_cache_new_block_size
+            engine.scheduler.num_gpu_blocks -= given
     model.is_layer_quant_list[layer_id] = False
     model.layer_quant_list.remove(layer_id)
     model.next_unquantized_layer = layer_id

@@ -13,8 +13,7 @@ Same ``BlockManager`` and bookkeeping as ``ElasticKVPool``.
 from __future__ import annotations
 
 import ctypes as C
-import time
-from typing import Optional, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -91,104 +90,68 @@ class LayerArena(_Arena):
 
 class VmmKVPool(ElasticKVPool):
     """``num_blocks`` blocks now, room for ``max_blocks``; sizes move in multiples of
-    ``chunk_blocks`` (one physical allocation per chunk and per tensor)."""
+    ``chunk_blocks`` (one physical allocation per chunk and per tensor).
+
+    ``placement="groups"`` (the default) lets ``mkv_arena_pair_grow`` choose the physical memory: K chunks
+    from one memory group of the device and V chunks from another, told apart by a store-rate measurement
+    at creation and at every growth (chunks of 256 MiB per tensor and more; smaller ones cannot be measured
+    and grow in the driver's order).  ``placement="plain"`` always takes the driver's order."""
 
     def __init__(self, num_blocks: int, max_blocks: int, num_layers: int, num_kv_heads: int, block_size: int,
                  head_dim: int, max_seqs_in_block_table: int, max_blocks_per_seq: int, chunk_blocks: int = 64,
-                 device: str = "cuda", settle_seconds: Optional[float] = None,
-                 v_stagger_bytes: Optional[int] = None):
+                 device: str = "cuda", v_stagger_bytes: int = 0, placement: str = "groups",
+                 placement_budget_bytes: int = 0):
         """``v_stagger_bytes``: how far into its range the V tensor starts (a multiple of 4 KiB below the chunk
-        size; it costs one more mapped chunk).  ``None``: chosen by the probe of ``kv_placement`` for pools of
-        ``MIN_BYTES_TO_TUNE`` per tensor and more, 0 otherwise."""
+        size; it costs one more mapped chunk).  ``placement_budget_bytes``: the most device memory a growth may
+        hold at once while it looks for chunks of the right groups (0: all that is free but 4 GiB)."""
         _capi.lib()
+        if placement not in ("groups", "plain"):
+            raise ValueError('placement must be "groups" or "plain"')
         self.device = torch.device(device, torch.cuda.current_device()) if device == "cuda" else torch.device(device)
         self.shape_tail = (num_layers, num_kv_heads, block_size, head_dim)
         self.chunk_blocks = chunk_blocks
         if num_blocks % chunk_blocks or max_blocks % chunk_blocks or not 0 < num_blocks <= max_blocks:
             raise ValueError(f"num_blocks and max_blocks must be multiples of chunk_blocks ({chunk_blocks})")
         self.max_blocks = max_blocks
-        from . import kv_placement as KP
         chunk = chunk_blocks * self.block_bytes
-        l, h, b, d = self.shape_tail
-        probe_ok = (b == 16 and d == 128 and num_blocks >= KP.MIN_BLOCKS_TO_TUNE
-                    and num_blocks * self.block_bytes >= KP.MIN_BYTES_TO_TUNE)
-        choose = v_stagger_bytes is None and probe_ok and chunk > max(KP.CANDIDATE_OFFSETS)
-        if v_stagger_bytes is not None and (v_stagger_bytes < 0 or v_stagger_bytes % 4096 or v_stagger_bytes >= chunk):
+        if v_stagger_bytes < 0 or v_stagger_bytes % 4096 or v_stagger_bytes >= chunk:
             raise ValueError("v_stagger_bytes must be a multiple of 4096 below the chunk size")
-        self._v_off = int(v_stagger_bytes or 0)
-        self._v_pad = chunk if (choose or self._v_off) else 0      # the V range is mapped one chunk further
+        self.placement = placement
+        self.placement_budget_bytes = int(placement_budget_bytes)
+        self._v_off = int(v_stagger_bytes)
+        self._v_pad = chunk if self._v_off else 0            # the V range is mapped one chunk further
         self._k_arena = _Arena(max_blocks * self.block_bytes, chunk)
         self._v_arena = _Arena(max_blocks * self.block_bytes + self._v_pad, chunk)
         self.k_cache_new, self.v_cache_new = [], []          # never used: the pool is one tensor
         self.kv_cache_new_block_size = 0
-        self.kv_placement = {"v_offset_bytes": 0, "tuned": False}     # two reservations: nothing to choose
+        self.kv_placement: Dict = {"v_offset_bytes": self._v_off, "placement": placement, "growths": []}
         self.block_manager = BlockManager("GPU", num_blocks, max_seqs_in_block_table, max_blocks_per_seq,
-                                          block_size, device=device)
+                                          block_size, device=device, reserve_blocks=max_blocks)
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
         self._map(num_blocks)
         self._zero(0, num_blocks)
-        self._settle(num_blocks, settle_seconds)
-        if choose:
-            self._choose_stagger(num_blocks)
-
-    def _choose_stagger(self, num_blocks: int) -> None:
-        """The K-to-V stagger of ``kv_placement``: the V tensor viewed at each candidate offset of its (zeroed) range,
-        the fastest kept unless offset 0 is within the probe's noise of it."""
-        from . import kv_placement as KP
-        probe, layers, probe_bytes = KP._make_probe(num_blocks, self.shape_tail, self.device, 0)
-        shape = (num_blocks, *self.shape_tail)
-        _capi.check(_capi.lib().mkv_fill_zero(self._v_arena.base + num_blocks * self.block_bytes, self._v_pad,
-                                              _capi.current_stream()))
-        timings = {off: float("inf") for off in KP.CANDIDATE_OFFSETS}
-        for _ in range(3):
-            for off in KP.CANDIDATE_OFFSETS:
-                v = torch.as_tensor(_RawDeviceMemory(self._v_arena.base + off, shape, self._v_arena), device=self.device)
-                timings[off] = min(timings[off], KP._probe_us(self.k_cache, v, probe, layers))
-        best = min(timings, key=timings.get)
-        if timings[best] > 0.995 * timings[0]:
-            best = 0
-        self._v_off = best
-        self._make_views(num_blocks)
-        self.kv_placement = dict(self.kv_placement, v_offset_bytes=best, tuned=True,
-                                 probe_us_per_launch={str(k): round(v, 2) for k, v in timings.items()},
-                                 probe_GBs=round(probe_bytes / timings[best] / 1e3, 1))
-
-    def _settle(self, num_blocks: int, settle_seconds: Optional[float]) -> None:
-        """``allocate_kv_caches``' one retry for mapped memory: a large pool whose probe reads recycled memory is
-        unmapped, the call sleeps and maps it again (the K-to-V stagger has no counterpart here: both ranges start
-        on a chunk boundary)."""
-        from . import kv_placement as KP
-        pool_bytes = 2 * num_blocks * self.block_bytes
-        if settle_seconds is None:
-            settle_seconds = KP.SETTLE_SECONDS
-        l, h, b, d = self.shape_tail
-        big = num_blocks * self.block_bytes >= KP.MIN_BYTES_TO_TUNE and num_blocks >= KP.MIN_BLOCKS_TO_TUNE
-        if not (big and b == 16 and d == 128 and settle_seconds > 0):
-            return
-        first = KP.probe_gather_GBs(self.k_cache, self.v_cache)
-        self.kv_placement = {"v_offset_bytes": 0, "tuned": False, "probe_GBs": first}
-        if first >= KP.settle_threshold_GBs(pool_bytes):
-            return
-        torch.cuda.synchronize(self.device)
-        self.k_cache = self.v_cache = None
-        self._k_arena.resize(0)
-        self._v_arena.resize(0)                              # the extra chunk of a staggered V range included
-        time.sleep(settle_seconds)
-        self._map(num_blocks)
-        self._zero(0, num_blocks)
-        self.kv_placement = {"v_offset_bytes": 0, "tuned": False,
-                             "probe_GBs": KP.probe_gather_GBs(self.k_cache, self.v_cache),
-                             "settled": {"first_probe_GBs": first, "waited_s": settle_seconds}}
 
     # -- mapping ---------------------------------------------------------------------
     def _map(self, num_blocks: int) -> None:
+        """Map (or unmap) so that both tensors hold ``num_blocks`` blocks."""
         nbytes = num_blocks * self.block_bytes
-        self._k_arena.resize(nbytes)
-        try:
-            self._v_arena.resize(nbytes + self._v_pad)
-        except Exception:
-            self._k_arena.resize(max(0, self._v_arena.mapped_bytes() - self._v_pad))
-            raise
+        k_have, v_have = self._k_arena.mapped_bytes(), self._v_arena.mapped_bytes()
+        k_add, v_add = nbytes - k_have, nbytes + self._v_pad - v_have
+        if self.placement == "groups" and k_add > 0 and v_add > 0:
+            info = _capi.MkvPairInfo()
+            rc = _capi.lib().mkv_arena_pair_grow(self._k_arena.handle, self._v_arena.handle, k_add, v_add,
+                                                 self.placement_budget_bytes, _capi.current_stream(), C.byref(info))
+            if rc == _capi.MKV_ENOSPC:
+                raise MemoryError("the device has no memory left for the pool to grow")
+            _capi.check(rc)
+            self.kv_placement["growths"].append({f: getattr(info, f) for f, _ in info._fields_ if f != "_pad"})
+        else:
+            self._k_arena.resize(nbytes)
+            try:
+                self._v_arena.resize(nbytes + self._v_pad)
+            except Exception:
+                self._k_arena.resize(k_have)
+                raise
         self._make_views(num_blocks)
 
     def _make_views(self, num_blocks: int) -> None:
@@ -224,10 +187,7 @@ class VmmKVPool(ElasticKVPool):
         self._zero(old, num_new_blocks)
         bm.num_blocks += num_new_blocks
         bm.num_free_blocks += num_new_blocks
-        new_map = torch.empty(bm.num_blocks, dtype=torch.bool, device=self.device)
-        new_map[:old] = bm.is_block_free
-        new_map[old:] = True
-        bm.is_block_free = new_map
+        bm.grow_free_map(num_new_blocks)
 
     def blocks_available_from(self, donor: "LayerArena", keep_bytes: int) -> int:
         """How many blocks ``expand_from(donor, keep_bytes)`` would add: the donor's mapped chunks behind
@@ -250,18 +210,33 @@ class VmmKVPool(ElasticKVPool):
             return 0
         nbytes = n * self.block_bytes
         torch.cuda.synchronize(self.device)                          # nothing may still use the donor's tail
+        have = self.block_manager.num_blocks
+        k_had, v_had = self._k_arena.mapped_bytes(), self._v_arena.mapped_bytes()
         self.k_cache = self.v_cache = None
-        donor.move_tail_to(self._k_arena, nbytes)
         try:
+            donor.move_tail_to(self._k_arena, nbytes)
             donor.move_tail_to(self._v_arena, nbytes)
         except Exception:
-            moved = self._k_arena.mapped_bytes() - self.block_manager.num_blocks * self.block_bytes
-            self._k_arena.move_tail_to(donor, moved)
-            self._make_views(self.block_manager.num_blocks)
+            # a move stops at the chunk that failed and leaves the earlier ones moved: hand back whatever
+            # either tensor received, so that the pool and the donor are as they were
+            self._give_back(donor, k_had, v_had)
+            self._make_views(have)
             raise
-        self._make_views(self.block_manager.num_blocks + n)
+        self._make_views(have + n)
         self._grew_by(n)
         return n
+
+    def _give_back(self, donor: "LayerArena", k_had: int, v_had: int) -> None:
+        """Return to ``donor`` the chunks the two arenas hold beyond ``k_had`` / ``v_had`` mapped bytes (V's
+        first, the reverse of the order they were taken in).  Best effort: a second failure is left to the
+        caller's exception."""
+        for arena, had in ((self._v_arena, v_had), (self._k_arena, k_had)):
+            extra = arena.mapped_bytes() - had
+            if extra > 0:
+                try:
+                    arena.move_tail_to(donor, extra)
+                except Exception:
+                    pass
 
     def shrink_into(self, donor: "LayerArena", new_num_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
         """``shrink_to(new_num_blocks)`` with the memory above the cut handed back to ``donor`` instead of
@@ -294,18 +269,39 @@ class VmmKVPool(ElasticKVPool):
             e = torch.empty(0, dtype=torch.int64, device=self.device)
             return e, e
         src, dst = self._relocate_live_blocks(new_num_blocks)        # synchronises the stream
-        bm.num_blocks -= removed
-        bm.num_free_blocks -= removed
-        bm.is_block_free = bm.is_block_free[:new_num_blocks].clone()
         torch.cuda.synchronize(self.device)                          # nothing may still read the tail
         if donor is None:
             self._map(new_num_blocks)
         else:
+            k_had, v_had = self._k_arena.mapped_bytes(), self._v_arena.mapped_bytes()
+            d_had = donor.mapped_bytes()
             self.k_cache = self.v_cache = None
-            self._v_arena.move_tail_to(donor, removed * self.block_bytes)
-            self._k_arena.move_tail_to(donor, removed * self.block_bytes)
+            try:
+                self._v_arena.move_tail_to(donor, removed * self.block_bytes)
+                self._k_arena.move_tail_to(donor, removed * self.block_bytes)
+            except Exception:
+                # take back what the donor received (K's chunks lie behind V's there), so that the pool still
+                # holds every block its counters speak of; the relocation stays (it is valid at either size)
+                self._take_back(donor, d_had, k_had, v_had)
+                self._make_views(bm.num_blocks)
+                raise
             self._make_views(new_num_blocks)
+        # the counters follow the memory: only now is the pool smaller
+        bm.num_blocks -= removed
+        bm.num_free_blocks -= removed
+        bm.shrink_free_map(new_num_blocks)
         return src, dst
+
+    def _take_back(self, donor: "LayerArena", d_had: int, k_had: int, v_had: int) -> None:
+        """Undo a partial hand-over to ``donor``: chunks it received beyond ``d_had`` return to the arenas that
+        are short of ``k_had`` / ``v_had`` (K's were mapped last, so they come back first).  Best effort."""
+        for arena, had in ((self._k_arena, k_had), (self._v_arena, v_had)):
+            short = had - arena.mapped_bytes()
+            if short > 0 and donor.mapped_bytes() - d_had >= short:
+                try:
+                    donor.move_tail_to(arena, short)
+                except Exception:
+                    pass
 
     # the segment-based entry points of the parent do not apply
     def tail_segment_unused(self) -> bool:

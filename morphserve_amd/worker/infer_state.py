@@ -175,7 +175,9 @@ class StepStateBuilder:
             self._copied[slot] = ev
         seq_ids, seq_lengths = dev[o_ids:o_ids + B], dev[o_len:o_len + B]
         if block_manager is not None and not ignore_kvcache:
-            block_manager.allocate_blocks_for_seqs(seq_ids, seq_lengths)
+            # the lists are at hand: the manager sizes and checks the request on the host and nothing waits
+            block_manager.allocate_blocks_for_seqs(seq_ids, seq_lengths, seq_ids_host=host[o_ids:o_ids + B],
+                                                   target_lens_host=host[o_len:o_len + B])
         dec = [int(x) for x in decoding_seq_lens_list]
         sbs, nsb = select_seq_block_size(self.num_kv_heads, dec)
         positions = dev[o_pos:o_pos + T]

@@ -51,11 +51,23 @@ def gather_allocated_blocks_and_unset(
     block_table: torch.Tensor,
     seq_ids: torch.Tensor,
     is_block_free: torch.Tensor,
+    total: int = None,
 ) -> torch.Tensor:
     """As the release above, and returns the released ids (int32, sequence-major,
-    logical block order).  One host read of the total sizes the result."""
+    logical block order).  One host read of the total sizes the result -- unless the
+    caller knows ``total`` (the sum of the rows' counts): then the result has its size
+    from the start and nothing is read back."""
     assert seq_ids.dtype == torch.int32 and seq_ids.is_contiguous()
     dev = block_table.device
+    if total is not None:
+        out = torch.empty(int(total), dtype=torch.int32, device=dev)
+        result = torch.empty(2, dtype=torch.int64, device=dev)
+        _capi.check(_capi.lib().mkv_bt_gather_release(
+            num_seq_allocated_blocks.data_ptr(), num_seq_allocated_blocks.shape[0],
+            block_table.data_ptr(), block_table.shape[1], seq_ids.data_ptr(), seq_ids.shape[0],
+            is_block_free.data_ptr(), int(is_block_free.shape[0]), out.data_ptr(), int(total), result.data_ptr(),
+            _capi.current_stream()))
+        return out
     cap = int(is_block_free.shape[0])
     out = torch.empty(cap, dtype=torch.int32, device=dev)
     result = torch.zeros(2, dtype=torch.int64, device=dev)

@@ -37,6 +37,31 @@ class KVSwapper:
         self.v_swap = torch.zeros(shape, dtype=torch.float16, device="cpu", pin_memory=pinned)
         self.pinned = pinned
         self.block_swap = 0          # blocks moved so far (model.py:478)
+        # (sequence ids | lengths) of a call travel to the device through pinned staging, two buffers in turn
+        rows = bm.block_table.shape[0]
+        on_gpu = pool.device.type == "cuda"
+        self._stage_host = [torch.empty((2, rows), dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]
+        self._stage_dev = [torch.empty((2, rows), dtype=torch.int32, device=pool.device) for _ in range(2)]
+        self._stage_done = [None, None]
+        self._stage_turn = 0
+
+    def _stage(self, ids_host, lens_host):
+        """Device views of the two lists, copied asynchronously from pinned memory on the current stream."""
+        n = len(ids_host)
+        if n > self._stage_host[0].shape[1]:
+            raise ValueError("more sequences than the block table has rows")
+        slot = self._stage_turn
+        self._stage_turn ^= 1
+        if self._stage_done[slot] is not None:
+            self._stage_done[slot].synchronize()             # the copy that last read this buffer (long finished)
+        host, dev = self._stage_host[slot], self._stage_dev[slot]
+        host.numpy()[0, :n] = ids_host
+        host.numpy()[1, :n] = lens_host
+        dev[:, :n].copy_(host[:, :n], non_blocking=True)
+        if dev.is_cuda:
+            self._stage_done[slot] = torch.cuda.Event()
+            self._stage_done[slot].record()
+        return dev[0, :n], dev[1, :n]
 
     def _swap(self, seq_ids_list: Sequence[int], is_swap_in: bool, use_kernel: Optional[bool] = None) -> int:
         if use_kernel is None:
@@ -45,10 +70,14 @@ class KVSwapper:
             raise ValueError("the one-kernel route needs a pinned swap space (pinned=True)")
         src_mgr = self.cpu_block_manager if is_swap_in else self.gpu_block_manager
         dst_mgr = self.gpu_block_manager if is_swap_in else self.cpu_block_manager
-        seq_ids = torch.tensor(list(seq_ids_list), dtype=torch.int32, device=self.pool.device)
-        seq_lengths = src_mgr.get_num_allocated_blocks(seq_ids) * self.gpu_block_manager.block_size
-        src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids)          # int32, sequence-major
-        dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths)     # int64, lowest free ids
+        ids_host = list(seq_ids_list)
+        # block counts from the managers' host copies: the id lists get their sizes without a device read
+        # (model.py:481-489 reads them back three times)
+        lens_host = src_mgr.host_num_allocated_blocks(ids_host) * self.gpu_block_manager.block_size
+        seq_ids, seq_lengths = self._stage(ids_host, lens_host)
+        src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids, seq_ids_host=ids_host)    # int32, sequence-major
+        dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths, seq_ids_host=ids_host,
+                                                   target_lens_host=lens_host)             # int64, lowest free ids
         n = int(src_ids.numel())
         assert int(dst_ids.numel()) == n
         self.block_swap += n
@@ -61,8 +90,9 @@ class KVSwapper:
                 src_ids.to(torch.int64).data_ptr(), dst_ids.data_ptr(), n, 1 if is_swap_in else 0,
                 C.byref(desc), self.k_swap.data_ptr(), self.v_swap.data_ptr(), self.k_swap.shape[0],
                 _capi.current_stream()))
-            # the temporaries above must outlive the launch; the stream is the caller's
-            torch.cuda.current_stream().synchronize()
+            # Nothing waits here: the id tensors are torch allocations on this stream, which hands their
+            # memory to later work of the same stream only; like the reference's asynchronous copies
+            # (block_swapping.cpp:51-80) the blocks have arrived once the stream has reached this point.
         else:
             desc = self.pool.descriptor()
             cnt = C.c_int64(0)
@@ -82,6 +112,7 @@ class KVSwapper:
         return self._swap(seq_ids_list, False, use_kernel)
 
     def free_seqs_resources(self, seq_ids_list: List[int]) -> None:
-        seq_ids = torch.tensor(list(seq_ids_list), dtype=torch.int32, device=self.pool.device)
-        self.gpu_block_manager.free_blocks_for_seqs(seq_ids)
-        self.cpu_block_manager.free_blocks_for_seqs(seq_ids)
+        ids_host = list(seq_ids_list)
+        seq_ids, _ = self._stage(ids_host, [0] * len(ids_host))
+        self.gpu_block_manager.free_blocks_for_seqs(seq_ids, seq_ids_host=ids_host)
+        self.cpu_block_manager.free_blocks_for_seqs(seq_ids, seq_ids_host=ids_host)

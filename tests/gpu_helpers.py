@@ -50,6 +50,7 @@ def load_manager(case: Case, dev) -> BlockManager:
     bm.num_seq_allocated_blocks.copy_(torch.from_numpy(case.n_alloc))
     bm.is_block_free.copy_(torch.from_numpy(case.is_free))
     bm.num_free_blocks = int(case.is_free.sum())
+    bm.invalidate_host_counts()                     # the counts were written behind the manager's back
     return bm
 
 

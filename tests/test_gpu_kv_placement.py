@@ -69,26 +69,5 @@ def test_elastic_pool_records_its_placement(cuda):
     plain = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda",
                           tune_placement=False)
     assert plain.kv_placement == {"v_offset_bytes": 0, "tuned": False} and plain.v_cache.storage_offset() == 0
-    small = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda")
-    assert small.kv_placement == {"v_offset_bytes": 0, "tuned": False}      # 128 MiB per tensor: left alone by default
-
-
-def test_retry_after_a_wait_when_the_probe_reads_low(cuda, monkeypatch):
-    """The one retry of pool creation: with the threshold above anything the probe can read the pool is given
-    back, the call waits ``settle_seconds`` and allocates once more; the result is an ordinary zeroed pool and the
-    record says what happened.  With 0 seconds (or a threshold of 0) nothing is retried."""
-    import time
-
-    from morphserve_amd import kv_placement as KP
-    tail = (2, 8, 16, 128)
-    monkeypatch.setattr(KP, "SETTLE_BELOW_GBS", 1e12)
-    t0 = time.perf_counter()
-    k, v, info = allocate_kv_caches(4096, tail, cuda, tune=True, settle_seconds=0.3)
-    assert time.perf_counter() - t0 >= 0.3
-    assert info["tuned"] and info["settled"]["waited_s"] == 0.3 and info["settled"]["first_probe_GBs"] > 0
-    assert info["probe_GBs"] > 0 and not k.any() and not v.any() and v.is_contiguous()
-    k2, v2, info2 = allocate_kv_caches(4096, tail, cuda, tune=True, settle_seconds=0)
-    assert "settled" not in info2
-    monkeypatch.setattr(KP, "SETTLE_BELOW_GBS", 0.0)
-    k3, v3, info3 = allocate_kv_caches(4096, tail, cuda, tune=True, settle_seconds=5.0)
-    assert "settled" not in info3
+    default = ElasticKVPool(4096, 1, 8, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8, device="cuda")
+    assert default.kv_placement == {"v_offset_bytes": 0, "tuned": False}    # the probe is opt-in
