@@ -9,10 +9,20 @@ token per sequence to the paged cache, then paged decode attention.
 Prints ONE JSON line: whole-step throughput in algorithmic HBM GB/s (inputs
 resident in HBM), the roofline of the dominant kernel (decode attention phase 1,
 timed per launch with HIP events on its own stream) and a CPU baseline (the
-oracle's torch-CPU statement of the same path on a bounded sample).
+oracle's torch-CPU statement of the same path on a bounded sample).  The default
+line also carries the pool resize of config 3 (``"resize"``), measured in the same
+process.
 
-``--workload cfg3_resize`` measures the elastic pool instead: grow 32k -> 96k
+``--workload cfg3_resize`` measures the elastic pool alone: grow 32k -> 96k
 blocks (zero fill), scatter ~24.5k live blocks, shrink to 40k with migration.
+``--workload placement_ab`` creates, measures (decode and resize) and frees pools
+with and without memory-group placement several times in ONE process, at once
+and after a pause: the evidence that the figures do not hang on allocation history.
+
+The pool is a ``VmmKVPool`` with K and V placed in different memory groups of the
+device (``--pool-backing torch`` / ``--placement plain`` give the other layouts).
+Everything that is timed runs on ``libmorphkv.so``; per-kernel breakdowns of steps
+that launch several kernels go through its diagnostic twin and are labelled so.
 """
 from __future__ import annotations
 
@@ -58,8 +68,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2_llama3_8b_decode",
                     choices=["cfg2_llama3_8b_decode", "cfg1_llama2_7b_layer", "cfg5_codellama34b_decode", "cfg3_resize",
-                             "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "copy_calibration", "mfma_calibration",
-                             "eviction", "prefill_shapes", "placement_probe", "timeline", "layer_handover", "step_state", "slab_gather"])
+                             "cfg4_mixed", "cfg4_serving", "cfg5_pressure_shrink", "placement_ab", "copy_calibration",
+                             "mfma_calibration", "eviction", "prefill_shapes", "layer_handover", "step_state",
+                             "allocator"])
     ap.add_argument("--pool-blocks", type=int, default=0, help="0 = the workload's own pool size")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--unfused", action="store_true",
@@ -75,38 +86,32 @@ def parse_args():
     ap.add_argument("--tables", choices=["permuted", "identity"], default="permuted",
                     help="decode workloads: block tables dealt from a seeded permutation of the pool (the "
                          "benchmark's definition) or in id order (diagnostic only)")
-    ap.add_argument("--vmm-chunk-blocks", type=int, default=64,
-                    help="with --pool-backing vmm: blocks per physical allocation (must divide the pool size)")
-    ap.add_argument("--pool-backing", choices=["torch", "vmm"], default="torch",
-                    help="decode workloads: the pool is a torch allocation (default) or one tensor over HIP "
-                         "virtual memory (VmmKVPool)")
-    ap.add_argument("--force-split", type=int, nargs=2, default=None, metavar=("TOKENS", "SPLITS"),
-                    help="decode workloads, diagnostic: split decomposition with exactly this split length and count")
+    ap.add_argument("--pool-backing", choices=["vmm", "torch"], default="vmm",
+                    help="the pool is one tensor over HIP virtual memory whose physical chunks the library places "
+                         "(VmmKVPool, default) or two torch allocations plus segments (ElasticKVPool)")
+    ap.add_argument("--placement", choices=["groups", "plain"], default="groups",
+                    help="with --pool-backing vmm: K and V chunks from different memory groups of the device "
+                         "(default) or in the order the driver hands them out")
+    ap.add_argument("--vmm-chunk-blocks", type=int, default=0,
+                    help="with --pool-backing vmm: blocks per physical allocation (must divide the pool size; "
+                         "0 = the largest divisor that keeps a chunk at or under 1 GiB per tensor)")
+    ap.add_argument("--v-stagger-bytes", type=int, default=0,
+                    help="with --pool-backing vmm: how far into its range the V tensor starts (a multiple of 4096)")
+    ap.add_argument("--no-wipe-wait", action="store_true",
+                    help="decode workloads, diagnostic: start measuring right after pool creation instead of waiting for "
+                         "the driver to wipe the candidate memory that creation gave back")
+    ap.add_argument("--ab-pause", type=float, default=10.0,
+                    help="placement_ab workload: seconds between the second free and the third allocation")
     ap.add_argument("--prefill-shapes", default="8x512,4x4096,2x8192,1x16384",
                     help="prefill_shapes workload: comma-separated SEQSxTOKENS prompt batches; SEQSxTOKENS+PREFIX is a "
                          "batch of chunks over PREFIX tokens already in a paged cache")
-    ap.add_argument("--no-placement-tuning", action="store_true",
-                    help="decode workloads, diagnostic: the V pool starts at its allocation's base (no probing of offsets)")
-    ap.add_argument("--settle-seconds", type=float, default=None,
-                    help="decode workloads: how long pool creation waits before its one retry when the placement probe "
-                         "reads a recently recycled allocation (default: the library's 12 s; 0 = never retry)")
-    ap.add_argument("--prefill-kv-heads", type=int, default=32,
-                    help="prefill_shapes workload, whole prompts: kv heads behind the 32 q heads (1 = every q head reads the "
-                         "same K/V, which then always comes out of the L2s: the same matrix work without the K/V traffic)")
-    ap.add_argument("--timeline-decode", default="64x1024-1536,1x32768,16x2048",
-                    help="timeline workload: comma-separated BATCHxLO-HI decode batches (config-2 model)")
-    ap.add_argument("--seq-order", choices=["drawn", "snake"], default="drawn",
-                    help="decode workloads, diagnostic: keep the drawn order of context lengths, or hand the batch over "
-                         "sorted so that slots 256 / Hkv apart (the two workgroups of a CU) hold a long and a short one")
-    ap.add_argument("--probe-clock-steps", type=int, default=150,
-                    help="placement_probe workload: decode steps run while the clocks are sampled (0 keeps a counter "
-                         "run down to the per-pool launches)")
     ap.add_argument("--prefill-data", choices=["randn", "zeros"], default="randn",
                     help="prefill_shapes workload: N(0,1) inputs (default) or all-zero inputs -- the same instruction "
                          "stream without switching activity in the matrix pipe, to show what the power limit costs")
-    ap.add_argument("--prefill-variants", default="0,4,8",
+    ap.add_argument("--prefill-variants", default="0",
                     help="prefill_shapes workload: workgroup shapes to time (0 = the library's own choice by prompt "
-                         "length, 4 = four waves / 128 query rows, 8 = eight waves / 256 query rows)")
+                         "length, on the product library; 4 = four waves / 128 query rows, 8 = eight waves / 256 query "
+                         "rows: forced through the diagnostic twin)")
     ap.add_argument("--seed", type=int, default=2)
     args = ap.parse_args()
     if args.ctx is None:
@@ -121,6 +126,67 @@ def decode_bytes_per_layer(lens, n, hq, hkv, d, b):
     attn = int(lens.sum()) * 2 * hkv * d * 2 + 2 * n * hq * d * 2 + int(((lens + b - 1) // b).sum()) * 4
     append = 2 * (n * 2 * hkv * d * 2)            # read k, v rows + write them into the cache
     return attn, append
+
+
+def auto_chunk_blocks(num_blocks, bytes_per_block_and_tensor):
+    """The largest divisor of num_blocks whose chunk stays at or under 1 GiB per tensor."""
+    target = max(1, (1 << 30) // bytes_per_block_and_tensor)
+    for c in range(min(target, num_blocks), 0, -1):
+        if num_blocks % c == 0:
+            return c
+    return 1
+
+
+def make_pool(args, num_blocks, max_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq):
+    """The KV pool of a workload by --pool-backing / --placement; (pool, description)."""
+    from morphserve_amd import ElasticKVPool, VmmKVPool
+    if args.pool_backing == "vmm":
+        per_tensor = L * HKV * B * D * 2
+        chunk = args.vmm_chunk_blocks or auto_chunk_blocks(int(np.gcd(num_blocks, max_blocks)), per_tensor)
+        pool = VmmKVPool(num_blocks, max_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, chunk_blocks=chunk,
+                         placement=args.placement, v_stagger_bytes=args.v_stagger_bytes)
+        what = (f"VmmKVPool, chunks of {chunk} blocks ({chunk * per_tensor / 2**20:.0f} MiB per tensor), placement "
+                f"{args.placement}")
+    else:
+        pool = ElasticKVPool(num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, reserve_blocks=max_blocks)
+        what = "ElasticKVPool: two torch allocations, growth by segments"
+    return pool, what
+
+
+WIPE_SECONDS_PER_GIB = 0.04
+
+
+def wait_for_driver_wipe(pool):
+    """Pool creation with memory-group placement gives the candidate chunks it did not keep back to the driver,
+    and the driver wipes released memory in the background (about 30 ms per GiB on this system; an allocation
+    that needs such memory waits for it, which is how the rate shows).  While that runs every kernel is a few
+    per cent slower, so a measurement that starts right after pool creation would time the driver's wipe, not
+    the pool.  A server creates its pool long before the first request; the benchmark waits here, for a time
+    computed from the bytes released (nothing is measured or compared to decide it).  Returns the seconds waited."""
+    released = sum(g.get("released_bytes", 0) for g in pool.kv_placement.get("growths", []))
+    wait = released / 2 ** 30 * WIPE_SECONDS_PER_GIB
+    if wait > 0:
+        time.sleep(wait)
+    return round(wait, 2)
+
+
+def diag_kernel_times(fn, kernel_ids):
+    """{kernel id: (launches, total ms)} of one pass of fn() routed through the DIAGNOSTIC twin of the library,
+    which brackets every launch of the listed kernels with an event pair (same sources, same kernels; the
+    figures that are reported as results are always timed on the product library)."""
+    import torch
+    from morphserve_amd import _capi
+    with _capi.use_diag_library():
+        _capi.prof_reset()
+        _capi.prof_enable(True)
+        try:
+            fn()
+            torch.cuda.synchronize()
+            out = {kid: _capi.prof_collect(kid) for kid in kernel_ids}
+        finally:
+            _capi.prof_enable(False)
+            _capi.prof_reset()
+    return out
 
 
 def _balanced_order():
@@ -150,14 +216,6 @@ def bench_decode(args):
     if args.batch:
         N = args.batch
     lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
-    if args.seq_order == "snake":                 # diagnostic: the batch arrives with long and short sequences alternating
-        run = max(1, 256 // HKV)                  # in runs of 256 / Hkv slots, the order that puts one of each on a CU
-        srt = np.sort(lens)[::-1]
-        out = srt.copy()
-        for r in range(len(srt) // run):
-            if r & 1:
-                out[r * run:(r + 1) * run] = srt[r * run:(r + 1) * run][::-1]
-        lens = out.astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     num_blocks = args.pool_blocks or default_blocks
     max_blocks_per_seq = max(128, -(-args.ctx[1] // B))
@@ -176,17 +234,13 @@ def bench_decode(args):
     live = perm[:pos].copy()
 
     shape = (num_blocks, L, HKV, B, D)
-    if args.pool_backing == "vmm":                # one tensor over HIP virtual memory
-        from morphserve_amd import VmmKVPool
-        vmm_pool = VmmKVPool(num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq,
-                             chunk_blocks=args.vmm_chunk_blocks, settle_seconds=args.settle_seconds)
-        k_cache, v_cache = vmm_pool.k_cache, vmm_pool.v_cache
-        kv_placement = vmm_pool.kv_placement
-    else:                                         # as ElasticKVPool creates them: two zeroed allocations, the V base
-        from morphserve_amd.kv_placement import allocate_kv_caches   # a few KiB in where the gather measures faster
-        k_cache, v_cache, kv_placement = allocate_kv_caches(num_blocks, shape[1:], dev, zero_init=True,
-                                                            tune=False if args.no_placement_tuning else None,
-                                                            settle_seconds=args.settle_seconds)
+    t_pool = time.perf_counter()
+    kv_pool, pool_what = make_pool(args, num_blocks, num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq)
+    torch.cuda.synchronize()
+    pool_creation_s = time.perf_counter() - t_pool
+    wiped_s = 0.0 if args.no_wipe_wait else wait_for_driver_wipe(kv_pool)
+    k_cache, v_cache = kv_pool.k_cache, kv_pool.v_cache
+    kv_placement = kv_pool.kv_placement
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     live_t = torch.from_numpy(live).to(dev)
@@ -203,10 +257,6 @@ def bench_decode(args):
     model = Cfg(num_layers=L, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D)
     engine = Cfg(block_size=B, max_blocks_per_seq=max_blocks_per_seq)
     st = build_infer_state([], seq_ids.tolist(), lens.tolist(), HKV, D)
-    if args.force_split:
-        from morphserve_amd.worker.kernels import paged_attn as PA
-        PA.SPLIT_POLICY = "reference"
-        st.seq_block_size, st.num_seq_blocks = args.force_split
 
     def new_step():
         # a serving loop builds its infer_state per step: what the wrappers keep on it (the balanced row
@@ -307,22 +357,19 @@ def bench_decode(args):
     other_ms = (time.perf_counter() - t0) * 1e3 / reps
 
     # -- dominant kernel: per-launch duration with HIP events on its stream -------------
-    # every launch bracketed by its own event pair (the pair's own cost included) ...
-    _capi.prof_reset()
-    _capi.prof_enable(True)
-    for _ in range(3):
-        step()
-    torch.cuda.synchronize()
-    launches, total_ms = _capi.prof_collect(_capi.K_ATTN_PHASE1)
-    p2_launches, p2_ms = _capi.prof_collect(_capi.K_ATTN_PHASE2)
-    ap_launches, ap_ms = _capi.prof_collect(_capi.K_APPEND_DECODE)
-    _capi.prof_enable(False)
-    _capi.prof_reset()
+    # Which kernels a step launches, and each one's share, from one pass through the diagnostic twin
+    # (every launch bracketed by its own event pair, the pair's own cost included) ...
+    def three_steps():
+        for _ in range(3):
+            step()
+    kt = diag_kernel_times(three_steps, (_capi.K_ATTN_PHASE1, _capi.K_ATTN_PHASE2, _capi.K_APPEND_DECODE))
+    (launches, total_ms), (p2_launches, p2_ms), (ap_launches, ap_ms) = (
+        kt[_capi.K_ATTN_PHASE1], kt[_capi.K_ATTN_PHASE2], kt[_capi.K_APPEND_DECODE])
     bracketed_ms = total_ms / max(launches, 1)
-    # ... and, when a step is nothing but launches of that kernel (fused call, one
-    # split), one event pair around whole steps: elapsed / launches
+    # ... and, when a step is nothing but launches of that kernel (fused call, one split), the figure that
+    # is reported: one event pair around whole steps of the PRODUCT library, elapsed / launches
     phase1_ms = bracketed_ms
-    timing = "event pair around every launch"
+    timing = "event pair around every launch (diagnostic twin of the library)"
     if not args.unfused and p2_launches == 0 and ap_launches == 0:
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
@@ -356,19 +403,18 @@ def bench_decode(args):
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {L} layers, GQA {HQ}q/{HKV}kv, head_dim 128, block 16, "
                                f"batch {N}, ctx U[{args.ctx[0]},{args.ctx[1]}], pool {num_blocks} blocks "
-                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), {args.tables} tables"
-                               + (", pool over HIP virtual memory" if args.pool_backing == "vmm" else ""),
+                               f"({num_blocks * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB), {args.tables} tables",
+                   "pool": pool_what,
                    "calls_per_layer": "store_kvcache + paged_attention (2 calls)" if args.unfused
                                       else "decode_append_and_attend (1 fused launch)",
                    "timed_as": "eager launches" if graph is None else "HIP graph replay of one step",
                    "row_order": ("the grid takes the batch's rows in the balanced order, computed once per step "
                                  "inside the timed region" if _balanced_order() and getattr(st, "_morphkv_decode_order", None)
                                  else "the grid takes the rows as given (a split batch needs no order)" if _balanced_order()
-                                 else "the grid takes the rows as given")
-                                + (", lengths handed over pre-ordered (--seq-order snake)" if args.seq_order == "snake" else ""),
-                   "pool_creation": "outside the timed region; the library's default: a short gather probe picks the V "
-                                    "pool's start and, when it reads memory the driver is still recycling, the pool is "
-                                    "allocated once more after a wait (see kv_placement: v_offset_bytes, probe_GBs, settled)"},
+                                 else "the grid takes the rows as given"),
+                   "pool_creation": f"outside the timed region, {pool_creation_s:.2f} s (kv_placement says what the "
+                                    f"memory-group measurement found), then {wiped_s} s for the driver to wipe the "
+                                    "candidate memory that creation gave back"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "kv_placement": kv_placement,
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
@@ -403,6 +449,10 @@ def bench_decode(args):
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_decode(k_cache, v_cache, live, table, seq_ids, lens, q, k_new, v_new,
                                                   HQ, HKV, D, B, attn_bytes + append_bytes, L)
+    del graph, k_cache, v_cache
+    if hasattr(kv_pool, "close"):
+        torch.cuda.synchronize()
+        kv_pool.close()                           # the memory goes back to the driver before the next workload
     return out
 
 
@@ -506,9 +556,10 @@ def _warm_resize_kernels(dev, L, HKV, B, D):
     assert src.numel() == 24
 
 
-def bench_resize(args):
+def bench_resize(args, with_cpu_baseline=True):
+    """Config 3: grow 32k -> 96k blocks of 2 MiB in eight steps (zero fill), scatter 24.5k live blocks over
+    the 96k range, shrink to 40k: plan, migration copy, block-table rewrite, release of the tail."""
     import torch
-    from morphserve_amd import ElasticKVPool, _capi
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -516,18 +567,21 @@ def bench_resize(args):
     ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1          # 32k -> 96k -> 40k blocks of 2 MiB
     rng = np.random.default_rng(args.seed)
     _warm_resize_kernels(dev, L, HKV, B, D)
-    pool = ElasticKVPool(ORG, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256,
-                         tune_placement=False if args.no_placement_tuning else None, settle_seconds=args.settle_seconds)
-    blk_bytes = pool.block_bytes
-    _capi.prof_reset()
-    _capi.prof_enable(True)
+    t0 = time.perf_counter()
+    if not args.vmm_chunk_blocks:
+        args = argparse.Namespace(**{**vars(args), "vmm_chunk_blocks": SEG})     # one physical allocation per segment and tensor
+    pool, pool_what = make_pool(args, ORG, ORG + NSEG * SEG, L, HKV, B, D, 512, 256)
     torch.cuda.synchronize()
+    create_s = time.perf_counter() - t0
+    pool.time_kernels = True
+    blk_bytes = pool.block_bytes
+    pool.fill_ms()                                     # drop the base pool's own zero fill from the record
     t0 = time.perf_counter()
     for _ in range(NSEG):
         pool.expand(SEG)
     torch.cuda.synchronize()
     expand_s = time.perf_counter() - t0
-    fz_launches, fz_ms = _capi.prof_collect(_capi.K_FILL_ZERO)
+    fz_ms = pool.fill_ms()
     grown = NSEG * SEG
     fill_gbs = grown * 2 * blk_bytes / (fz_ms * 1e-3) / 1e9
 
@@ -557,33 +611,44 @@ def bench_resize(args):
     src, dst = pool.shrink_to(new_n)
     torch.cuda.synchronize()
     shrink_s = time.perf_counter() - t0
-    mg_launches, mg_ms = _capi.prof_collect(_capi.K_MIGRATE)
-    _capi.prof_enable(False)
-    _capi.prof_reset()
+    mg_ms = pool.last_migrate_ms
     moves = int(src.numel())
     assert moves == moves_expected
+    # what the caller waits for before the pool is usable again: plan + copy + table rewrite + sync; giving the
+    # tail's memory back to the driver (unmapping the chunks / freeing the segments) follows it
+    relocate_s = getattr(pool, "last_relocate_s", None) or shrink_s
     moved_bytes = moves * 2 * blk_bytes
     traffic = 2 * moved_bytes                          # read + write
     achieved = traffic / (mg_ms * 1e-3) / 1e9
-    whole = traffic / shrink_s / 1e9
+    whole = traffic / relocate_s / 1e9
+    kv_placement = pool.kv_placement
+    del src, dst
+    if hasattr(pool, "close"):
+        pool.close()
     cpu = None
-    if not args.no_cpu_baseline:
+    if with_cpu_baseline and not args.no_cpu_baseline:
         cpu = cpu_baseline_resize(rng)
     return {
         **({"cpu_baseline": cpu} if cpu else {}),
         "metric": "pool resize + live-block migration HBM GB/s (read+write), 1 MI355X",
         "value": round(whole, 1), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 0,
-        "ms_per_step": round(shrink_s * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(relocate_s * 1e3, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"cfg3_resize: 2 MiB blocks (32 layers x 8 kv heads x 16 x 128 fp16, K+V), "
-                               f"grow {ORG}->{total} (zero fill), {len(live)} live scattered, shrink to {new_n}"},
-        "moves": moves, "moved_GiB": round(moved_bytes / 2 ** 30, 2), "kv_placement": pool.kv_placement,
+                               f"grow {ORG}->{total} (zero fill), {len(live)} live scattered, shrink to {new_n}",
+                   "pool": pool_what,
+                   "timed": "shrink_to up to the point where every live block has its new place and the table is "
+                            "rewritten (plan + migration copy + table rewrite + stream sync); shrink_ms_with_release "
+                            "adds the release of the memory above the cut"},
+        "moves": moves, "moved_GiB": round(moved_bytes / 2 ** 30, 2), "kv_placement": kv_placement,
+        "pool_creation_s": round(create_s, 3),
         "expand_s": round(expand_s, 4), "zero_fill_GBs": round(fill_gbs, 1),
+        "shrink_ms_with_release": round(shrink_s * 1e3, 3),
         "pct_of_hbm_peak": round(100 * whole / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic(f"cfg3_resize moves={moves}"),
-                     "avg_launch_ms": round(mg_ms / max(mg_launches, 1), 4),
+                     "avg_launch_ms": round(mg_ms, 4),
                      "algorithmic_bytes_per_launch": traffic},
     }
 
@@ -593,21 +658,26 @@ def bench_pressure_shrink(args):
     mid-run the scheduler's own give-back rule releases 25 % of the blocks (63 578 -> 47 684)
     while a quarter of the live blocks sit above the cut and have to move."""
     import torch
-    from morphserve_amd import ElasticKVPool, _capi, build_infer_state, decode_append_and_attend, paged_attention
+    from morphserve_amd import build_infer_state, decode_append_and_attend, paged_attention
     from morphserve_amd.server import PoolEngine, Request, Scheduler
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L, HQ, HKV, D, B, N = 48, 64, 8, 128, 16, 128
     KEEP, SEG = 47684, 15894                       # 63 578 blocks of 3 MiB (K+V) = 186 GiB
+    if args.pool_backing == "vmm":                 # whole chunks of 512 blocks (768 MiB per tensor): 63 488 -> 47 616
+        KEEP, SEG = 47616, 15872
+        if not args.vmm_chunk_blocks:
+            args = argparse.Namespace(**{**vars(args), "vmm_chunk_blocks": 512})
     total = KEEP + SEG
     rng = np.random.default_rng(args.seed)
     lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
     nblk = (lens.astype(np.int64) + B - 1) // B
     max_seqs, max_bps = 256, 128
     _warm_resize_kernels(dev, L, HKV, B, D)
-    pool = ElasticKVPool(KEEP, L, HKV, B, D, max_seqs_in_block_table=max_seqs, max_blocks_per_seq=max_bps)
+    pool, pool_what = make_pool(args, KEEP, total, L, HKV, B, D, max_seqs, max_bps)
     pool.expand(SEG)
+    pool.time_kernels = True
     perm = rng.permutation(total)
     seq_ids = rng.permutation(max_seqs)[:N].astype(np.int32)
     table = np.full((max_seqs, max_bps), -1, dtype=np.int32)
@@ -628,8 +698,10 @@ def bench_pressure_shrink(args):
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
     tail = (L, HKV, B, D)
-    for ids, kt, vt, off in ((live[live < KEEP], pool.k_cache, pool.v_cache, 0),
-                             (live[live >= KEEP], pool.k_cache_new[0], pool.v_cache_new[0], KEEP)):
+    parts = (((live, pool.k_cache, pool.v_cache, 0),) if not pool.k_cache_new else
+             ((live[live < KEEP], pool.k_cache, pool.v_cache, 0),
+              (live[live >= KEEP], pool.k_cache_new[0], pool.v_cache_new[0], KEEP)))
+    for ids, kt, vt, off in parts:
         idt = torch.from_numpy(ids - off).to(dev)
         for c0 in range(0, len(ids), 128):
             idx = idt[c0:c0 + 128]
@@ -684,16 +756,13 @@ def bench_pressure_shrink(args):
     engine.scheduler = sched
     for i in range(N):
         sched.running_q.append(Request(prompt_len=int(lens[i]) - 1, output_len=1, request_id=int(seq_ids[i])))
-    _capi.prof_reset()
-    _capi.prof_enable(True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     sched.get_next_batch(engine)
     torch.cuda.synchronize()
     shrink_ms = (time.perf_counter() - t0) * 1e3
-    mg_launches, mg_ms = _capi.prof_collect(_capi.K_MIGRATE)
-    _capi.prof_enable(False)
-    _capi.prof_reset()
+    mg_ms = pool.last_migrate_ms or 0.0
+    relocate_ms = (pool.last_relocate_s or 0.0) * 1e3
     assert pool.num_blocks == KEEP and not pool.k_cache_new and sched.num_gpu_blocks == KEEP, "no give-back happened"
     moves = engine.migrated_blocks
     assert moves == int((live >= KEEP).sum())
@@ -713,13 +782,15 @@ def bench_pressure_shrink(args):
         "warmup": args.warmup, "ms_per_step": round(after_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"cfg5_pressure_shrink: 48 layers, GQA 64q/8kv, batch {N}, ctx U[{args.ctx[0]},"
-                               f"{args.ctx[1]}], pool {total} -> {KEEP} blocks of 3 MiB, eager launches"},
+                               f"{args.ctx[1]}], pool {total} -> {KEEP} blocks of 3 MiB, eager launches",
+                   "pool": pool_what},
         "ms_per_step_before": round(before_ms, 4), "ms_per_step_after": round(after_ms, 4),
         "pct_of_hbm_peak_before": round(100 * step_bytes / (before_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "pct_of_hbm_peak_after": round(100 * step_bytes / (after_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "shrink": {"decided_by": "Scheduler.get_next_batch -> try_quant2org -> quant2org_and_update_kvcache(migrate)",
-                   "ms": round(shrink_ms, 3), "live_blocks_moved": moves, "moved_GiB": round(moved / 2 ** 30, 2),
-                   "GBs_read_plus_write": round(2 * moved / (shrink_ms * 1e-3) / 1e9, 1),
+                   "ms": round(shrink_ms, 3), "relocation_ms": round(relocate_ms, 3),
+                   "live_blocks_moved": moves, "moved_GiB": round(moved / 2 ** 30, 2),
+                   "GBs_read_plus_write": round(2 * moved / (max(relocate_ms, 1e-9) * 1e-3) / 1e9, 1),
                    "migrate_kernel_ms": round(mg_ms, 3),
                    "attention_outputs_bit_identical_across_shrink": identical},
         "roofline": {"bound": "hbm", "kernel": "pool_migrate_kernel",
@@ -810,18 +881,12 @@ def bench_mixed(args):
 
     ms_per_step = time_steps(step)
     ms_two_streams = time_steps(step_two_streams)
-    _capi.prof_reset()
-    _capi.prof_enable(True)
-    step()
-    torch.cuda.synchronize()
-    avg = {}
-    for name, kid in (("prefill_attn", _capi.K_PREFILL_ATTN), ("append_prefill", _capi.K_APPEND_PREFILL),
-                      ("append_decode", _capi.K_APPEND_DECODE), ("attn_phase1", _capi.K_ATTN_PHASE1),
-                      ("attn_phase2", _capi.K_ATTN_PHASE2)):
-        cnt, ms = _capi.prof_collect(kid)
-        avg[name] = ms / cnt if cnt else None
-    _capi.prof_enable(False)
-    _capi.prof_reset()
+    # the step's kernels one by one: a pass through the diagnostic twin, every launch bracketed by an event pair
+    names = (("prefill_attn", _capi.K_PREFILL_ATTN), ("append_prefill", _capi.K_APPEND_PREFILL),
+             ("append_decode", _capi.K_APPEND_DECODE), ("attn_phase1", _capi.K_ATTN_PHASE1),
+             ("attn_phase2", _capi.K_ATTN_PHASE2))
+    kt = diag_kernel_times(step, [kid for _, kid in names])
+    avg = {name: (kt[kid][1] / kt[kid][0] if kt[kid][0] else None) for name, kid in names}
 
     # the step before the append: rotary embedding of q and k, separate or fused with it
     from morphserve_amd import rotary_embedding_and_store_kvcache, rotary_embedding_inplace, rotary_tables
@@ -1060,7 +1125,7 @@ def bench_mfma_calibration(args):
     g.manual_seed(args.seed)
     data = torch.randn(64 * 1024, dtype=torch.float16, device=dev, generator=g)
     sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
-    lib = _capi.lib()
+    lib = _capi.diag_lib()                     # the calibration loop lives in the diagnostic twin
     iters = 2000
     out = {}
     for mode, name in ((0, "registers_constant_operands"), (1, "registers_normal_operands"), (2, "lds_normal_operands")):
@@ -1092,8 +1157,8 @@ def bench_prefill_shapes(args):
     import torch
     from morphserve_amd import _capi
 
+    import contextlib
     dev = torch.device("cuda:0")
-    lib = _capi.lib()
     H, D = 32, 128
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
@@ -1105,7 +1170,7 @@ def bench_prefill_shapes(args):
         body, _, pfx = shape.partition("+")
         prefix = int(pfx) if pfx else 0
         paged = pfx != ""
-        HKV = H if paged else args.prefill_kv_heads
+        HKV = H
         nseq, ln = (int(x) for x in body.split("x"))
         T = nseq * ln
         if args.prefill_data == "zeros":
@@ -1137,41 +1202,45 @@ def bench_prefill_shapes(args):
             prefix_t = torch.full((nseq,), prefix, dtype=torch.int32, device=dev)
         outs, row = {}, {}
         for var in variants:
-            _capi.check(lib.mkv_set_prefill_variant(var))
-            o = torch.full_like(q, float("nan"))
+            # 0 = the product library and its own choice; a forced shape exists in the diagnostic twin only
+            with (_capi.use_diag_library() if var else contextlib.nullcontext(_capi.lib())) as lib:
+                if var:
+                    _capi.check(lib.mkv_set_prefill_variant(var))
+                o = torch.full_like(q, float("nan"))
 
-            def run():
-                if paged:
-                    chunked_prefill_attention(q, k_cache, v_cache, [], [], bt, model, engine, st, 0, o, prefix_t, prefix)
-                else:
-                    _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                                     starts.data_ptr(), lens.data_ptr(), nseq, ln, H, HKV, D, D ** -0.5,
-                                                     _capi.current_stream()))
-            # warm up by time, not by count: after the set-up kernels (random fills) the first few tens of
-            # milliseconds of matrix work run at another clock, and a timing taken there reads 10-15 % low
-            t_warm = time.perf_counter()
-            n_warm = 0
-            while n_warm < max(args.warmup, 1) or time.perf_counter() - t_warm < 0.06:
-                run()
-                n_warm += 1
-                if n_warm % 8 == 0:
-                    torch.cuda.synchronize()
-            torch.cuda.synchronize()
-            reps = max(args.steps, 5)
-            blocks = []
-            for _ in range(3):                       # median of three timed blocks of `reps` launches
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(reps):
+                def run():
+                    if paged:
+                        chunked_prefill_attention(q, k_cache, v_cache, [], [], bt, model, engine, st, 0, o, prefix_t, prefix)
+                    else:
+                        _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                         starts.data_ptr(), lens.data_ptr(), nseq, ln, H, HKV, D, D ** -0.5,
+                                                         _capi.current_stream()))
+                # warm up by time, not by count: after the set-up kernels (random fills) the first few tens of
+                # milliseconds of matrix work run at another clock, and a timing taken there reads 10-15 % low
+                t_warm = time.perf_counter()
+                n_warm = 0
+                while n_warm < max(args.warmup, 1) or time.perf_counter() - t_warm < 0.06:
                     run()
-                e1.record()
+                    n_warm += 1
+                    if n_warm % 8 == 0:
+                        torch.cuda.synchronize()
                 torch.cuda.synchronize()
-                blocks.append(e0.elapsed_time(e1) / reps)
-            ms = sorted(blocks)[1]
-            outs[var] = o
-            row[f"variant_{var}"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
-                                     "frac_of_2500": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4)}
-        _capi.check(lib.mkv_set_prefill_variant(0))
+                reps = max(args.steps, 5)
+                blocks = []
+                for _ in range(3):                       # median of three timed blocks of `reps` launches
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(reps):
+                        run()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    blocks.append(e0.elapsed_time(e1) / reps)
+                ms = sorted(blocks)[1]
+                outs[var] = o
+                row[f"variant_{var}"] = {"us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
+                                         "frac_of_2500": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4)}
+                if var:
+                    _capi.check(lib.mkv_set_prefill_variant(0))
         base = outs[variants[0]].float()
         assert torch.isfinite(base).all()
         row["max_abs_diff_between_variants"] = max(float((outs[x].float() - base).abs().max()) for x in variants)
@@ -1182,259 +1251,12 @@ def bench_prefill_shapes(args):
             "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": best["us"] / 1e3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
             "data": "synthetic",
-            "config": {"workload": f"prefill_shapes: 32 q / {args.prefill_kv_heads} kv heads, head_dim 128, prompt batches {args.prefill_shapes}, "
+            "config": {"workload": f"prefill_shapes: 32 q / 32 kv heads, head_dim 128, prompt batches {args.prefill_shapes}, "
                                    f"workgroup shapes {args.prefill_variants}, inputs {args.prefill_data}"},
             "shapes": rows,
             "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel",
                          "achieved": best["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
                          "frac": round(best["TFLOPs"] / 2500.0, 4), "traffic": None}}
-
-
-def bench_timeline(args):
-    """Where a launch's time goes, per workgroup: the attention kernels stamp the GPU's 100 MHz counter at
-    fixed points of every workgroup's life (mkv_diag_timeline); this workload runs ONE stamped launch per
-    shape -- prefill batches (--prefill-shapes, whole prompts only) and decode batches (--timeline-decode,
-    BATCHxLO-HI on the config-2 model, fused append, rows in the balanced order) -- and reports, in
-    microseconds from the first workgroup's entry, the distribution of each point, of the phases between
-    them, and of the moment each CU is done (workgroups w and w + 256 share a CU while a grid is one round of
-    two workgroups per CU)."""
-    import ctypes as C
-    import torch
-    from morphserve_amd import _capi
-    from morphserve_amd.worker.kernels.paged_attn import choose_split
-
-    dev = torch.device("cuda:0")
-    lib = _capi.lib()
-    P = 8
-    g = torch.Generator(device=dev)
-    g.manual_seed(args.seed)
-
-    def q3(x):
-        x = x.double()
-        return {"min": round(float(x.min()), 2), "p10": round(float(x.quantile(0.1)), 2),
-                "median": round(float(x.median()), 2), "p90": round(float(x.quantile(0.9)), 2),
-                "max": round(float(x.max()), 2)}
-
-    def stamped(run, nwg, names, phases):
-        for _ in range(5):
-            run()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(20):
-            run()
-        e1.record()
-        torch.cuda.synchronize()
-        buf = torch.zeros(nwg * P, dtype=torch.int64, device=dev)
-        _capi.check(lib.mkv_diag_timeline(buf.data_ptr(), nwg))
-        try:
-            run()                          # the stamping instance's own first launch (code load) is not the one kept
-            torch.cuda.synchronize()
-            buf.zero_()
-            run()
-            torch.cuda.synchronize()
-        finally:
-            _capi.check(lib.mkv_diag_timeline(None, 0))
-        d = buf.cpu().view(nwg, P).double()
-        d = d[d[:, 0] > 0]
-        t0 = d[:, 0].min()
-        row = {"us_per_launch_unstamped": round(e0.elapsed_time(e1) / 20 * 1e3, 2), "workgroups": int(d.shape[0])}
-        row["points_us"] = {nm: q3((d[d[:, k] > 0, k] - t0) / 100.0) for k, nm in enumerate(names) if (d[:, k] > 0).any()}
-        row["phases_us"] = {}
-        for a, b, nm in phases:
-            m = (d[:, a] > 0) & (d[:, b] > 0)
-            if m.any():
-                row["phases_us"][nm] = q3((d[m, b] - d[m, a]) / 100.0)
-        last = d.max(dim=1).values
-        fin = (last - t0) / 100.0
-        row["workgroup_done_us"] = {"mean": round(float(fin.mean()), 2), "max": round(float(fin.max()), 2)}
-        if d.shape[0] == 512:
-            cu = torch.maximum(fin[:256], fin[256:])
-            row["cu_done_us"] = {**q3(cu), "mean": round(float(cu.mean()), 2)}
-            row["cu_done_mean_us_by_xcd"] = [round(float(cu[x::8].mean()), 2) for x in range(8)]
-        return row
-
-    rows = {}
-    H, D = 32, 128
-    for shape in [x for x in args.prefill_shapes.split(",") if x and "+" not in x]:
-        nseq, ln = (int(x) for x in shape.split("x"))
-        T = nseq * ln
-        q, k, v = (torch.randn((T, H, D), dtype=torch.float16, device=dev, generator=g) for _ in range(3))
-        o = torch.empty_like(q)
-        starts = torch.arange(nseq, dtype=torch.int32, device=dev) * ln
-        lens = torch.full((nseq,), ln, dtype=torch.int32, device=dev)
-
-        def run():
-            _capi.check(lib.mkv_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), starts.data_ptr(),
-                                             lens.data_ptr(), nseq, ln, H, H, D, D ** -0.5, _capi.current_stream()))
-        names = ["entry", "first tile staged", "tiles done", "written", "second part: first tile staged",
-                 "second part: tiles done", "second part: written"]
-        phases = [(0, 1, "entry -> first tile staged"), (1, 2, "first part: key tiles"), (2, 3, "first part: output"),
-                  (2, 4, "first part done -> second part staged"), (4, 5, "second part: key tiles"),
-                  (5, 6, "second part: output")]
-        rows["prefill " + shape] = stamped(run, 1 << 16, names, phases)
-        del q, k, v, o
-
-    L, HQ, HKV, B = 32, 32, 8, 16
-    nb = args.pool_blocks or 16384
-    kc = torch.randn((nb, L, HKV, B, D), dtype=torch.float16, device=dev, generator=g)
-    vc = torch.randn((nb, L, HKV, B, D), dtype=torch.float16, device=dev, generator=g)
-    pool = _capi.make_pool(kc, vc)
-    rng = np.random.default_rng(args.seed)
-    for shape in [x for x in args.timeline_decode.split(",") if x]:
-        n_s, ctx = shape.split("x")
-        N = int(n_s)
-        lo, hi = (int(x) for x in ctx.split("-")) if "-" in ctx else (int(ctx), int(ctx))
-        lens = rng.integers(lo, hi + 1, size=N).astype(np.int32)
-        nblk = (lens + B - 1) // B
-        mbs = int(nblk.max()) + 1
-        assert int(nblk.sum()) <= nb, "pool too small for this batch"
-        perm = rng.permutation(nb)
-        table = np.zeros((N, mbs), dtype=np.int32)
-        pos = 0
-        for i in range(N):
-            table[i, :nblk[i]] = perm[pos:pos + nblk[i]]
-            pos += nblk[i]
-        bt = torch.from_numpy(table).to(dev)
-        lens_t = torch.from_numpy(lens).to(dev)
-        ids = torch.arange(N, dtype=torch.int32, device=dev)
-        q = torch.randn((N, HQ, D), dtype=torch.float16, device=dev, generator=g)
-        kn = torch.randn((N, HKV, D), dtype=torch.float16, device=dev, generator=g)
-        vn = torch.randn((N, HKV, D), dtype=torch.float16, device=dev, generator=g)
-        tps, splits = choose_split(N, HKV, int(lens.max()), B)
-        mid_o = torch.empty(N * HQ * splits * D, dtype=torch.float32, device=dev)
-        mid_lse = torch.empty(N * HQ * splits, dtype=torch.float32, device=dev)
-        order = torch.empty(N, dtype=torch.int32, device=dev)
-        o = torch.empty((N, HQ * D), dtype=torch.float16, device=dev)
-        if N >= 2:
-            _capi.check(lib.mkv_decode_order(lens_t.data_ptr(), N, HKV, order.data_ptr(), _capi.current_stream()))
-
-        def run():
-            _capi.check(lib.mkv_decode_attn_ordered(
-                q.data_ptr(), o.data_ptr(), C.byref(pool), bt.data_ptr(), mbs, ids.data_ptr(), lens_t.data_ptr(),
-                order.data_ptr() if N >= 2 else None, N, HQ, D ** -0.5, 5, tps, splits, mid_o.data_ptr(),
-                mid_lse.data_ptr(), kn.data_ptr(), vn.data_ptr(), None, None, _capi.current_stream()))
-        names = ["entry", "before the block loop", "blocks done", "stored"]
-        phases = [(0, 1, "entry -> block loop"), (1, 2, "block loop"), (2, 3, "merge of the waves and store")]
-        row = stamped(run, splits * HKV * N, names, phases)
-        row["splits"] = splits
-        row["note"] = "us_per_launch_unstamped includes the merge launch when splits > 1"
-        row["algorithmic_MB"] = round(sum(decode_bytes_per_layer(lens, N, HQ, HKV, D, B)) / 1e6, 1)
-        rows["decode " + shape] = row
-    first = next(iter(rows.values()))
-    return {"metric": "per-workgroup timeline of the attention kernels, 1 MI355X", "value": first["us_per_launch_unstamped"],
-            "unit": "us/launch", "n_gpus": 1, "steps": 1, "warmup": 5, "ms_per_step": first["us_per_launch_unstamped"] / 1e3,
-            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
-            "data": "synthetic",
-            "config": {"workload": f"timeline: prefill {args.prefill_shapes} (MHA 32/32), decode {args.timeline_decode} "
-                                   f"(config-2 model, pool {nb} blocks); one stamped launch each"},
-            "shapes": rows}
-
-
-def bench_placement_probe(args):
-    """Does the rate follow the ALLOCATION?  Four KV pools of 32 GiB in one process, the same config-2 decode
-    batch (same tables, same q / k / v) run on each in turn, twice; then a sequential 1 GiB copy inside each
-    pool (the migration kernel on consecutive block ids: streaming, hardly any address translation).
-    Per pool: microseconds per decode layer and GB/s, copy GB/s.  Under `rocprofv3 --pmc` the decode
-    launches come in groups of 32 * (steps + 1) per (round, pool), in that order."""
-    import ctypes as C
-    import torch
-    from morphserve_amd import _capi
-
-    dev = torch.device("cuda:0")
-    L, HQ, HKV, D, B, N = 32, 32, 8, 128, 16, 64
-    n_pools, nb = 4, args.pool_blocks or 16384
-    reps = max(args.steps, 1)
-    rng = np.random.default_rng(args.seed)
-    lens = rng.integers(args.ctx[0], args.ctx[1] + 1, size=N).astype(np.int32)
-    nblk = (lens + B - 1) // B
-    perm = rng.permutation(nb)
-    table = np.full((256, 128), -1, dtype=np.int32)
-    seq_ids = rng.permutation(256)[:N].astype(np.int32)
-    pos = 0
-    for i in range(N):
-        table[seq_ids[i], :nblk[i]] = perm[pos:pos + nblk[i]]
-        pos += nblk[i]
-    bt, ids, ln = (torch.from_numpy(x).to(dev) for x in (table, seq_ids, lens))
-    g = torch.Generator(device=dev)
-    g.manual_seed(args.seed)
-    q = torch.randn((L, N, HQ, D), dtype=torch.float16, device=dev, generator=g)
-    kn = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
-    vn = torch.randn((L, N, HKV, D), dtype=torch.float16, device=dev, generator=g)
-    o = torch.empty((L, N, HQ, D), dtype=torch.float16, device=dev)
-    lib = _capi.lib()
-    stream = _capi.current_stream()
-    attn_bytes, _ = decode_bytes_per_layer(lens, N, HQ, HKV, D, B)
-    pools = []
-    for _ in range(n_pools):
-        k = torch.zeros((nb, L, HKV, B, D), dtype=torch.float16, device=dev)
-        v = torch.zeros((nb, L, HKV, B, D), dtype=torch.float16, device=dev)
-        pools.append((k, v, _capi.make_pool(k, v)))
-
-    def step(pool):
-        for layer in range(L):
-            _capi.check(lib.mkv_decode_append_attn(
-                kn[layer].data_ptr(), vn[layer].data_ptr(), q[layer].data_ptr(), o[layer].data_ptr(), C.byref(pool),
-                bt.data_ptr(), 128, ids.data_ptr(), ln.data_ptr(), N, HQ, float(D ** -0.5), layer, 1536, 1, None, None,
-                stream))
-
-    def timed(fn, n):
-        fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n
-
-    out = {"pools": []}
-    decode_us = [[0.0] * n_pools for _ in range(2)]
-    for rnd in range(2):
-        for p, (_, _, pool) in enumerate(pools):
-            decode_us[rnd][p] = timed(lambda: step(pool), reps) / L * 1e3
-    moves = 512
-    src = torch.arange(1024, 1024 + moves, dtype=torch.int64, device=dev)
-    dst = torch.arange(0, moves, dtype=torch.int64, device=dev)
-    moved = moves * 2 * (L * HKV * B * D * 2)
-    for p, (k, v, pool) in enumerate(pools):
-        ms = timed(lambda: _capi.check(lib.mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream)), 5)
-        out["pools"].append({"k_address": hex(k.data_ptr()), "v_address": hex(v.data_ptr()),
-                             "decode_us_per_layer": [round(decode_us[0][p], 2), round(decode_us[1][p], 2)],
-                             "decode_GBs": round(attn_bytes / (decode_us[1][p] * 1e-6) / 1e9, 1),
-                             "sequential_copy_GBs_read_plus_write": round(2 * moved / (ms * 1e-3) / 1e9, 1)})
-    # clocks while the decode kernel runs, read from sysfs (no child process: a program that has
-    # initialised the GPU must not start another one through fork + exec on some hosts)
-    import glob
-    import threading
-    got = {}
-
-    def ask():
-        for name in ("sclk", "mclk", "fclk"):
-            for path in sorted(glob.glob(f"/sys/class/drm/card*/device/pp_dpm_{name}")):
-                try:
-                    cur = [ln.split(":", 1)[1].strip(" *\n") for ln in open(path) if ln.rstrip().endswith("*")]
-                except OSError:
-                    continue
-                if cur:
-                    got[name] = cur[0]
-                    break
-    t = threading.Thread(target=ask)
-    t.start()
-    for _ in range(args.probe_clock_steps):
-        step(pools[0][2])
-    torch.cuda.synchronize()
-    t.join()
-    out["clocks_under_load"] = got or None
-    best = max(x["decode_GBs"] for x in out["pools"])
-    worst = min(x["decode_GBs"] for x in out["pools"])
-    return {"metric": "decode attention GB/s per pool allocation (same batch, one process)", "value": best, "unit": "GB/s",
-            "n_gpus": 1, "steps": reps, "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
-            "config": {"workload": f"placement_probe: {n_pools} pools of {nb} blocks ({nb * 2 * L * HKV * B * D * 2 / 2**30:.0f} GiB "
-                                   f"each), config-2 decode batch on each, fused launches, eager"},
-            "spread_pct": round(100.0 * (best - worst) / best, 2), **out, "roofline": None}
 
 
 def bench_copy_calibration(args):
@@ -1454,16 +1276,17 @@ def bench_copy_calibration(args):
     src = torch.arange(1024, 1024 + moves, dtype=torch.int64, device=dev)
     dst = torch.arange(0, moves, dtype=torch.int64, device=dev)
     stream = _capi.current_stream()
-    _capi.prof_reset()
-    _capi.prof_enable(True)
-    for _ in range(max(args.steps, 1)):
-        _capi.check(_capi.lib().mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream))
+    _capi.check(_capi.lib().mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream))
+    launches = max(args.steps, 1)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    launches, ms = _capi.prof_collect(_capi.K_MIGRATE)
-    _capi.prof_enable(False)
-    _capi.prof_reset()
+    e0.record()
+    for _ in range(launches):
+        _capi.check(_capi.lib().mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream))
+    e1.record()
+    torch.cuda.synchronize()
     moved = moves * 2 * (L * HKV * B * D * 2)
-    avg = ms / max(launches, 1)
+    avg = e0.elapsed_time(e1) / launches
     return {"metric": "plain device copy GB/s (read+write)", "value": round(2 * moved / (avg * 1e-3) / 1e9, 1),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 0, "ms_per_step": round(avg, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
@@ -1471,61 +1294,127 @@ def bench_copy_calibration(args):
             "bytes_read_per_launch": moved, "bytes_written_per_launch": moved}
 
 
-# ---------------------------------------------------------------------------------
-def bench_slab_gather(args):
-    """What the memory system gives the decode gather: random 4 KiB slab reads and nothing else (2 GiB per launch),
-    against the bytes in flight per CU, the footprint (one 64 GiB allocation or two) and which XCDs read which
-    allocation (``mkv_diag_slab_gather``)."""
+def bench_placement_ab(args):
+    """Does a figure depend on when and where its pool was allocated?  ONE process creates a pool, measures the
+    decode step of config 2 on it and the resize of config 3, and frees it -- for the memory-group placement
+    and for the plain order, three times each: at once, again at once, and after a pause (the driver hands
+    out different memory for some seconds after a large free).  Every figure of the table should sit on one
+    level per placement."""
+    import gc
     import torch
-    from morphserve_amd import _capi
+    rows = []
+    base = {**vars(args), "no_cpu_baseline": True, "no_resize": True, "pool_backing": "vmm",
+            "workload": "cfg2_llama3_8b_decode", "vmm_chunk_blocks": 0}
+    base["no_wipe_wait"] = False
+    schedule = [("first", 0.0), ("again at once", 0.0), (f"after {args.ab_pause:g} s", args.ab_pause)]
+    for when, pause in schedule:
+        for placement in ("groups", "plain", "groups, measured without waiting for the driver's wipe"):
+            if pause:
+                time.sleep(pause)
+            a = argparse.Namespace(**{**base, "placement": placement.split(",")[0],
+                                      "no_wipe_wait": "without waiting" in placement})
+            d = bench_decode(a)
+            gc.collect()
+            r = bench_resize(a, with_cpu_baseline=False)
+            gc.collect()
+            rows.append({"when": when, "placement": placement,
+                         "decode_pct_of_hbm_peak": d["pct_of_hbm_peak"], "decode_ms_per_step": d["ms_per_step"],
+                         "decode_kernel_frac": d["roofline"]["frac"],
+                         "resize_pct_of_hbm_peak": r["pct_of_hbm_peak"], "resize_ms": r["ms_per_step"],
+                         "migrate_kernel_frac": r["roofline"]["frac"], "zero_fill_GBs": r["zero_fill_GBs"],
+                         "decode_pool_creation": d["config"]["pool_creation"],
+                         "decode_pool_growths": d["kv_placement"]["growths"],
+                         "resize_pool_growths": r["kv_placement"]["growths"]})
+            print(json.dumps({k: v for k, v in rows[-1].items() if not k.endswith("growths")}), file=sys.stderr, flush=True)
+    g = [x for x in rows if x["placement"] == "groups"]
+    p = [x for x in rows if x["placement"] == "plain"]
+    return {"metric": "decode and resize, % of HBM peak, over repeated pool creations in one process", "unit": "%",
+            "value": min(x["decode_pct_of_hbm_peak"] for x in g), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": max(x["decode_ms_per_step"] for x in g), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16 / u8", "data": "synthetic",
+            "config": {"workload": "placement_ab: config 2 decode and config 3 resize on a VmmKVPool, memory-group "
+                                   "placement against the plain order, allocate -> measure -> free three times each"},
+            "range_with_groups": {"decode_pct": [min(x["decode_pct_of_hbm_peak"] for x in g), max(x["decode_pct_of_hbm_peak"] for x in g)],
+                                  "resize_pct": [min(x["resize_pct_of_hbm_peak"] for x in g), max(x["resize_pct_of_hbm_peak"] for x in g)]},
+            "range_plain": {"decode_pct": [min(x["decode_pct_of_hbm_peak"] for x in p), max(x["decode_pct_of_hbm_peak"] for x in p)],
+                            "resize_pct": [min(x["resize_pct_of_hbm_peak"] for x in p), max(x["resize_pct_of_hbm_peak"] for x in p)]},
+            "rows": rows}
+
+
+def bench_allocator(args):
+    """Launch times of the block manager's kernels on maps of config-2 and config-3 size (rocprofv3 --kernel-trace
+    gives the per-kernel durations of this workload), and the host time of allocate_blocks_for_seqs with and
+    without host lists."""
+    import torch
+    from morphserve_amd import BlockManager, ElasticKVPool
 
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    lib, stream = _capi.lib(), _capi.current_stream()
-    gib = 1 << 30
-    bufs = [torch.ones(64 * gib, dtype=torch.uint8, device=dev) for _ in range(2)]
-    spacer = torch.empty(32 * gib, dtype=torch.uint8, device=dev)
-    bufs.append(torch.ones(64 * gib, dtype=torch.uint8, device=dev))      # 96 GiB below the first one
-    del spacer
-    sink = torch.zeros(1, dtype=torch.int32, device=dev)
-    slabs = 64 * gib // 4096
-    per, total = 64, 1 << 19                                               # 2 GiB per launch
-
-    def rate(a, b, loads, wpc, by_xcd=0, mask=0):
-        def launch():
-            _capi.check(lib.mkv_diag_slab_gather(a.data_ptr(), b.data_ptr(), slabs, total // per, per, loads, wpc, by_xcd,
-                                                 mask, sink.data_ptr(), stream))
-        launch()
-        launch()
+    out = {}
+    rng = np.random.default_rng(args.seed)
+    for num_blocks, fill in ((65536, 0.08), (65536, 0.9), (98304, 0.25)):
+        bm = BlockManager("GPU", num_blocks, 512, 256, 16)
+        used = rng.random(num_blocks) < fill
+        bm.is_block_free.copy_(torch.from_numpy(~used))
+        bm.num_free_blocks = int((~used).sum())
+        ids = torch.arange(64, dtype=torch.int32, device=dev)
+        ids_h = list(range(64))
+        cur = np.zeros(64, dtype=np.int64)
+        times = {}
+        for mode in ("host lists", "device read"):
+            reps = max(args.steps, 20)
+            host_s = 0.0
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(reps):
+                cur += 16                                  # one more block per sequence
+                tgt = torch.from_numpy(cur.astype(np.int32)).to(dev)
+                t0 = time.perf_counter()
+                if mode == "host lists":
+                    bm.allocate_blocks_for_seqs(ids, tgt, seq_ids_host=ids_h, target_lens_host=cur)
+                else:
+                    bm.allocate_blocks_for_seqs(ids, tgt)
+                host_s += time.perf_counter() - t0
+            e1.record()
+            torch.cuda.synchronize()
+            times[mode] = {"host_us_per_call": round(host_s / reps * 1e6, 1),
+                           "stream_us_per_call_incl_input_copy": round(e0.elapsed_time(e1) / reps * 1e3, 1)}
+        out[f"{num_blocks} blocks, {int(fill * 100)} % used"] = times
+    # shrink planning on the config-3 map
+    pool = ElasticKVPool(64, 1, 1, 16, 128, max_seqs_in_block_table=8, max_blocks_per_seq=8)
+    bm = pool.block_manager
+    total, new_n = 98304, 40960
+    free = torch.ones(total, dtype=torch.bool, device=dev)
+    live = torch.from_numpy(rng.permutation(total)[:24576]).to(dev)
+    src = torch.empty(total - new_n, dtype=torch.int64, device=dev)
+    dst = torch.empty_like(src)
+    remap = torch.empty(total, dtype=torch.int32, device=dev)
+    res = torch.zeros(4, dtype=torch.int64, device=dev)
+    from morphserve_amd import _capi
+    reps = max(args.steps, 20)
+    tot_ms = 0.0
+    for _ in range(reps):
+        free.fill_(True)
+        free[live] = False
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(args.steps):
-            launch()
+        _capi.check(_capi.lib().mkv_pool_plan_shrink(free.data_ptr(), total, new_n, src.data_ptr(), dst.data_ptr(),
+                                                     total - new_n, remap.data_ptr(), res.data_ptr(),
+                                                     _capi.current_stream()))
         e1.record()
-        e1.synchronize()
-        return round(total * 4096 * args.steps / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
-
-    in_flight = {}
-    for tag, b in (("one allocation (64 GiB)", bufs[0]), ("two allocations (128 GiB)", bufs[1])):
-        in_flight[tag] = {f"{wpc} workgroups per CU x {loads} loads per thread = {wpc * 256 * loads * 16 // 1024} KiB per CU":
-                          rate(bufs[0], b, loads, wpc) for wpc in (1, 2, 4, 8) for loads in (1, 2, 4, 8)}
-    by_xcd = {}
-    for tag, b in (("second allocation = the neighbour", bufs[1]), ("second allocation = 96 GiB further down", bufs[2])):
-        by_xcd[tag] = {name: rate(bufs[0], b, 4, 8, 1, mask) for name, mask in
-                       (("all XCDs read the first", 0x00), ("all XCDs read the second", 0xFF),
-                        ("XCDs 0-3 the first, 4-7 the second", 0xF0), ("XCDs 0-3 the second, 4-7 the first", 0x0F),
-                        ("even XCDs the first, odd the second", 0xAA), ("XCDs 0,1,4,5 the first, 2,3,6,7 the second", 0xCC))}
-    best = max(in_flight["two allocations (128 GiB)"].values())
-    return {
-        "metric": "random 4 KiB slab reads, nothing else in the kernel, GB/s, 1 MI355X",
-        "value": best, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 2,
-        "ms_per_step": round(total * 4096 / best / 1e6, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "slab_gather: 2 GiB of random 4 KiB slabs per launch out of 64 GiB allocations"},
-        "GBs_by_bytes_in_flight": in_flight, "GBs_by_xcd_group": by_xcd,
-        "roofline": {"bound": "hbm", "kernel": "diag_slab_gather_kernel<U>", "achieved": best, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(best / HBM_PEAK_GBS, 4), "traffic": None},
-    }
+        torch.cuda.synchronize()
+        tot_ms += e0.elapsed_time(e1)
+    out["pool_plan_shrink 98304 -> 40960, 24576 live"] = {"event_us_per_launch": round(tot_ms / reps * 1e3, 1),
+                                                          "moves": int(res[0].item())}
+    del pool, bm
+    first = out["65536 blocks, 8 % used"]["host lists"]
+    return {"metric": "block manager: host microseconds per allocate_blocks_for_seqs call", "unit": "us",
+            "value": first["host_us_per_call"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": first["host_us_per_call"] / 1e3, "higher_is_better": False, "scaling": "weak",
+            "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+            "config": {"workload": "allocator: 64 decoding sequences take one more block each per call; free maps "
+                                   "of 65 536 and 98 304 entries"},
+            "cases": out}
 
 
 def bench_step_state(args):
@@ -1684,9 +1573,12 @@ def _eviction_routes(args, L, HKV, num_blocks, n_seq, blocks_per_seq):
     moved = n_seq * blocks_per_seq
     gbytes = moved * pool.block_bytes * 2 / 1e9
     results = {}
-    for name, pinned, use_kernel in (("kernel_pinned", True, True), ("memcpy_runs_pinned", True, False),
-                                     ("memcpy_runs_pageable", False, False)):
-        sw = KVSwapper(pool, moved + 64, pinned=pinned)
+    for name, pinned, use_kernel, cpu_tables in (("kernel_pinned", True, True, "device"),
+                                                 ("kernel_pinned_host_tables", True, True, "host"),
+                                                 ("memcpy_runs_pinned", True, False, "device"),
+                                                 ("memcpy_runs_pinned_host_tables", True, False, "host"),
+                                                 ("memcpy_runs_pageable", False, False, "device")):
+        sw = KVSwapper(pool, moved + 64, pinned=pinned, cpu_tables=cpu_tables)
         out_ms, in_ms = [], []
         for rep in range(max(args.warmup, 1) + args.steps):
             torch.cuda.synchronize()
@@ -1721,24 +1613,24 @@ def main():
     from morphserve_amd import _capi
     _capi.lib()
     table = {"cfg2_llama3_8b_decode": bench_decode, "cfg5_codellama34b_decode": bench_decode,
-             "cfg1_llama2_7b_layer": bench_decode,
-             "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
+             "cfg1_llama2_7b_layer": bench_decode, "cfg3_resize": bench_resize, "cfg4_mixed": bench_mixed,
+             "cfg4_serving": bench_serving, "cfg5_pressure_shrink": bench_pressure_shrink,
+             "placement_ab": bench_placement_ab, "allocator": bench_allocator,
              "copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration,
-             "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes, "placement_probe": bench_placement_probe,
-             "cfg5_pressure_shrink": bench_pressure_shrink, "cfg4_serving": bench_serving,
-             "timeline": bench_timeline, "layer_handover": bench_layer_handover, "step_state": bench_step_state, "slab_gather": bench_slab_gather}
+             "eviction": bench_eviction, "prefill_shapes": bench_prefill_shapes,
+             "layer_handover": bench_layer_handover, "step_state": bench_step_state}
     out = table[args.workload](args)
     if args.workload == "cfg2_llama3_8b_decode" and not args.no_resize and not args.pool_blocks:
-        # the second target of the path in the same process and the same JSON line: the decode pool is gone
-        # (its tensors were locals of bench_decode), the resize workload builds its own
+        # the second target of the path in the same process and the same JSON line: the decode pool has been
+        # closed, the resize workload builds its own
         import gc
         gc.collect()
-        torch.cuda.empty_cache()
         r = bench_resize(args)
         out["resize"] = {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"],
                          "unit": r["unit"], "ms": r["ms_per_step"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
                          "moves": r["moves"], "moved_GiB": r["moved_GiB"], "expand_s": r["expand_s"],
-                         "kv_placement": r["kv_placement"],
+                         "shrink_ms_with_release": r["shrink_ms_with_release"], "pool": r["config"]["pool"],
+                         "timed": r["config"]["timed"], "kv_placement": r["kv_placement"],
                          "zero_fill_GBs": r["zero_fill_GBs"], "dtype": r["dtype"], "roofline": r["roofline"],
                          **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})}
     print(json.dumps(out))

@@ -332,13 +332,17 @@ int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes);
  * destinations share a group and at 78 % when they do not, and the decode gather is fastest over a
  * pool that touches at most two groups.  mkv_arena_pair_grow maps k_add_bytes more at the end of
  * `k` and v_add_bytes more at the end of `v` (both arenas of one pool: same chunk size and device)
- * with K chunks from one group and V chunks from another: it creates candidate chunks (at most
- * budget_bytes of them at a time, 0 = all free device memory but 4 GiB), tells their groups apart by
- * the rate of a store-only kernel that fills a candidate and a reference side by side (a relative
- * measurement: no absolute rate is assumed, and a device without such groups yields one group and
- * the plain order), keeps what it needs, preferring each arena's own group, and gives the rest back.
- * Where an arena can still grow it also keeps one spare chunk of its group as the reference for the
- * next call (held until mkv_arena_destroy).  Chunks under 256 MiB cannot be measured: plain growth.
+ * with K chunks from one group and V chunks from another.  The call that creates the pool (both
+ * arenas empty) creates candidate chunks until it holds enough of two groups (at most budget_bytes
+ * of them at a time, 0 = all free device memory but 4 GiB), tells their groups apart by the rate of
+ * a store-only kernel that fills a candidate and a reference side by side (a relative measurement:
+ * no absolute rate is assumed, and a device without such groups yields one group and the plain
+ * order), keeps what it needs and gives the rest back (info->released_bytes: the driver wipes
+ * released memory in the background, about 30 ms per GiB, and kernels run a few per cent slower
+ * while it does).  Where an arena can still grow it also keeps one spare chunk of its group as the
+ * reference for later calls (held until mkv_arena_destroy); a later call creates exactly the chunks
+ * it needs, measures them against those references and gives each arena the ones of its own group
+ * first.  Chunks under 256 MiB cannot be measured: plain growth.
  * Host call; it synchronises `stream`, on which the measurement kernels run; the new memory holds
  * whatever the measurement left (the caller clears it, as after mkv_arena_resize).  MKV_ENOSPC when
  * the device has no memory left (nothing changed).  `info` (may be NULL) reports what was found. */
@@ -351,6 +355,7 @@ typedef struct mkv_pair_info {
     int32_t _pad;
     double probe_ms;        /* GPU time of the measurement */
     double total_ms;        /* host time of the call */
+    uint64_t released_bytes;/* candidate memory given back to the driver at the end of the call */
 } mkv_pair_info;
 int mkv_arena_pair_grow(mkv_arena* k, mkv_arena* v, uint64_t k_add_bytes, uint64_t v_add_bytes,
                         uint64_t budget_bytes, void* stream, mkv_pair_info* info);

@@ -56,6 +56,7 @@ class MkvPairInfo(C.Structure):
         ("_pad", C.c_int32),
         ("probe_ms", C.c_double),
         ("total_ms", C.c_double),
+        ("released_bytes", C.c_uint64),
     ]
 
 

@@ -14,6 +14,7 @@
 // never an absolute rate, so a device without such groups simply yields one group and the plain order.
 #include "common.h"
 
+#include <stdlib.h>
 #include <algorithm>
 #include <chrono>
 #include <vector>
@@ -341,16 +342,38 @@ static int map_ref(mkv_arena* a, hipMemGenericAllocationHandle_t h) {
     return MKV_OK;
 }
 
+// The purest of a few candidates: a chunk whose own two halves fill slowest lies in ONE group (a chunk
+// pieced together from two groups fills as fast as two chunks of different groups do, and would make
+// every other chunk look "different" if it were the reference).
+static int purest(PairGrow& g, const std::vector<size_t>& among, size_t* best, double* best_rate) {
+    *best = among[0];
+    *best_rate = 1e30;
+    for (size_t j = 0; j < among.size() && j < 6; ++j) {
+        double r = 0.0;
+        int rc = g.rate(g.cand[among[j]].va, g.cand[among[j]].va + g.probe_bytes, &r);
+        if (rc) return rc;
+        if (r < *best_rate) {
+            *best_rate = r;
+            *best = among[j];
+        }
+    }
+    return MKV_OK;
+}
+
 static int pair_grow(PairGrow& g, size_t need_k, size_t need_v, uint64_t budget_bytes, mkv_pair_info* info) {
     mkv_arena *k = g.k, *v = g.v;
     MKV_HIP(hipEventCreate(&g.e0));
     MKV_HIP(hipEventCreate(&g.e1));
     const size_t need = need_k + need_v;
-    // a spare per arena only where the arena can still grow afterwards
-    const bool k_wants_ref = !k->has_ref && (k->chunks.size() + need_k) * k->chunk < k->reserved;
-    const bool v_wants_ref = !v->has_ref && (v->chunks.size() + need_v) * v->chunk < v->reserved;
+    // Only the call that creates the pool searches for chunks of two groups, and keeps one spare of each as
+    // the references of later calls (where the arenas can still grow).  A later call measures the chunks the
+    // driver hands it against those references and deals them out as well as they allow, no more: looking
+    // further would mean creating and giving back memory the rest of the process may be waiting for.
+    const bool first = !k->has_ref && !v->has_ref && k->chunks.empty() && v->chunks.empty();
+    const bool k_wants_ref = first && (k->chunks.size() + need_k) * k->chunk < k->reserved;
+    const bool v_wants_ref = first && (v->chunks.size() + need_v) * v->chunk < v->reserved;
     const size_t spare = (k_wants_ref ? 1 : 0) + (v_wants_ref ? 1 : 0);
-    size_t budget_chunks = (size_t)(budget_bytes / g.chunk);
+    size_t budget_chunks = first ? (size_t)(budget_bytes / g.chunk) : 0;
     if (budget_chunks < need + spare) budget_chunks = need + spare;
 
     size_t got = 0;
@@ -360,73 +383,73 @@ static int pair_grow(PairGrow& g, size_t need_k, size_t need_v, uint64_t budget_
         set_error("the device has no memory left for %zu chunks of %llu bytes", need, (unsigned long long)g.chunk);
         return MKV_ENOSPC;
     }
-    // references: the arenas' spares, or (first call) two candidates that turn out to lie in different groups
+    // references: the arenas' spares, or (first call) candidates that turn out to lie in different groups
     char *ref_k = k->has_ref ? k->ref_va : nullptr, *ref_v = v->has_ref ? v->ref_va : nullptr;
     size_t first_unmeasured = 0;
     double self_k = 0.0;
-    if (!ref_k && !ref_v) {
-        ref_k = g.cand[0].va;
-        g.cand[0].group = 0;
-        rc = g.rate(ref_k, ref_k + g.probe_bytes, &self_k);
-        if (rc) return rc;
-        first_unmeasured = 1;
-    }
     int groups_found = 1;
     for (;;) {
         // measure what has not been measured yet
         const size_t lo = first_unmeasured, hi = g.cand.size();
+        if (!ref_k && !ref_v) {
+            std::vector<size_t> all;
+            for (size_t i = lo; i < hi; ++i) all.push_back(i);
+            size_t anchor = 0;
+            if ((rc = purest(g, all, &anchor, &self_k))) return rc;
+            ref_k = g.cand[anchor].va;
+            g.cand[anchor].group = 0;
+        }
         if (ref_k && ref_v) {
             // two references in different groups: a candidate's own two rates decide (same group ~ 3/4 of the other)
             for (size_t i = lo; i < hi; ++i) {
+                if (g.cand[i].group >= 0) continue;
                 double rk = 0, rv = 0;
                 if ((rc = g.rate(ref_k, g.cand[i].va, &rk)) || (rc = g.rate(ref_v, g.cand[i].va, &rv))) return rc;
                 g.cand[i].group = rk < 0.9 * rv ? 0 : (rv < 0.9 * rk ? 1 : 2);
             }
-            groups_found = 2;
-            for (auto& c : g.cand) if (c.group == 2) groups_found = 3;
-        } else if (ref_k || ref_v) {
+        } else {
             // one reference so far: split by the step in the rates against it
             char* ref = ref_k ? ref_k : ref_v;
             const int own = ref_k ? 0 : 1;
             if (self_k == 0.0 && (rc = g.rate(ref, ref + g.probe_bytes, &self_k))) return rc;
-            std::vector<double> r(hi - lo);
-            for (size_t i = lo; i < hi; ++i)
-                if ((rc = g.rate(ref, g.cand[i].va, &r[i - lo]))) return rc;
+            std::vector<size_t> idx;
+            for (size_t i = lo; i < hi; ++i) if (g.cand[i].group < 0) idx.push_back(i);
+            std::vector<double> r(idx.size());
+            for (size_t j = 0; j < idx.size(); ++j)
+                if ((rc = g.rate(ref, g.cand[idx[j]].va, &r[j]))) return rc;
             std::vector<char> same;
             split_by_rate(r, self_k, &same);
-            int other = -1;
-            for (size_t i = lo; i < hi; ++i) {
-                g.cand[i].group = same[i - lo] ? own : -2;       // -2: another group, not yet told which
-                if (!same[i - lo] && other < 0) other = (int)i;
+            std::vector<size_t> others;
+            for (size_t j = 0; j < idx.size(); ++j) {
+                if (same[j]) g.cand[idx[j]].group = own;
+                else others.push_back(idx[j]);
             }
-            if (other >= 0) {
-                // the first candidate of another group becomes the second reference; the rest of "another
+            if (!others.empty()) {
+                // the purest chunk of another group becomes the second reference; the rest of "another
                 // group" is measured against it
-                char* ref2 = g.cand[other].va;
-                (ref_k ? ref_v : ref_k) = ref2;
-                g.cand[other].group = 1 - own;
+                size_t second = 0;
                 double self2 = 0.0;
-                if ((rc = g.rate(ref2, ref2 + g.probe_bytes, &self2))) return rc;
-                std::vector<size_t> idx;
-                for (size_t i = 0; i < g.cand.size(); ++i) if (g.cand[i].group == -2) idx.push_back(i);
-                std::vector<double> r2(idx.size());
-                for (size_t j = 0; j < idx.size(); ++j)
-                    if ((rc = g.rate(ref2, g.cand[idx[j]].va, &r2[j]))) return rc;
+                if ((rc = purest(g, others, &second, &self2))) return rc;
+                char* ref2 = g.cand[second].va;
+                (ref_k ? ref_v : ref_k) = ref2;
+                g.cand[second].group = 1 - own;
+                std::vector<size_t> rest;
+                for (size_t i : others) if (i != second) rest.push_back(i);
+                std::vector<double> r2(rest.size());
+                for (size_t j = 0; j < rest.size(); ++j)
+                    if ((rc = g.rate(ref2, g.cand[rest[j]].va, &r2[j]))) return rc;
                 std::vector<char> same2;
                 split_by_rate(r2, self2, &same2);
-                groups_found = 2;
-                for (size_t j = 0; j < idx.size(); ++j) {
-                    g.cand[idx[j]].group = same2[j] ? 1 - own : 2;
-                    if (!same2[j]) groups_found = 3;
-                }
+                for (size_t j = 0; j < rest.size(); ++j) g.cand[rest[j]].group = same2[j] ? 1 - own : 2;
             }
         }
         first_unmeasured = hi;
-        // enough chunks of two different groups?  (the anchors can be used like any other candidate)
-        size_t n0 = 0, n1 = 0;
-        for (auto& c : g.cand) { n0 += c.group == 0; n1 += c.group == 1; }
+        size_t n0 = 0, n1 = 0, n2 = 0;
+        for (auto& c : g.cand) { n0 += c.group == 0; n1 += c.group == 1; n2 += c.group == 2; }
+        groups_found = 1 + (n1 > 0 || (ref_k && ref_v)) + (n2 > 0);
+        // enough chunks of two different groups?  (the references are candidates like any other)
         const size_t want_k = need_k + (k_wants_ref ? 1 : 0), want_v = need_v + (v_wants_ref ? 1 : 0);
-        const bool fits = (n0 >= want_k && n1 >= want_v) || (!k->has_ref && !v->has_ref && n1 >= want_k && n0 >= want_v);
+        const bool fits = (n0 >= want_k && n1 >= want_v) || (first && n1 >= want_k && n0 >= want_v);
         if (fits || g.cand.size() >= budget_chunks) break;
         size_t batch = std::min(budget_chunks - g.cand.size(), std::max<size_t>(need / 2, 8));
         if ((rc = g.more(batch, &got))) return rc;
@@ -435,7 +458,7 @@ static int pair_grow(PairGrow& g, size_t need_k, size_t need_v, uint64_t budget_
     // On a first call the two groups are interchangeable: K takes the one with more chunks.
     size_t n0 = 0, n1 = 0;
     for (auto& c : g.cand) { n0 += c.group == 0; n1 += c.group == 1; }
-    if (!k->has_ref && !v->has_ref && n1 > n0) {
+    if (first && n1 > n0) {
         for (auto& c : g.cand) if (c.group == 0 || c.group == 1) c.group = 1 - c.group;
         std::swap(n0, n1);
     }
@@ -488,6 +511,8 @@ static int pair_grow(PairGrow& g, size_t need_k, size_t need_v, uint64_t budget_
     if (spare_k >= 0 && ((rc = g.unstage(g.cand[spare_k])) || (rc = map_ref(k, g.cand[spare_k].h)))) g.cand[spare_k].taken = false;
     if (spare_v >= 0 && ((rc = g.unstage(g.cand[spare_v])) || (rc = map_ref(v, g.cand[spare_v].h)))) g.cand[spare_v].taken = false;
     if (info) {
+        size_t kept = need_k + need_v + (spare_k >= 0 ? 1 : 0) + (spare_v >= 0 ? 1 : 0);
+        info->released_bytes = (uint64_t)(g.cand.size() - kept) * g.chunk;
         info->groups_found = groups_found;
         info->candidates = (int32_t)g.cand.size();
         info->k_chunks = (int32_t)need_k;

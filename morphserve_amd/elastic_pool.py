@@ -10,6 +10,7 @@ plan (device scan) -> batched block copy -> block-table rewrite -> truncate.
 from __future__ import annotations
 
 import ctypes as C
+import time
 from typing import List, Optional, Tuple
 
 import torch
@@ -49,6 +50,35 @@ class ElasticKVPool:
                                           max_blocks_per_seq, block_size, device=device,
                                           reserve_blocks=reserve_blocks)
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
+        self._init_timing()
+
+    def _init_timing(self) -> None:
+        # measurement on request: with time_kernels set, the migration copy of a shrink and the zero fill of a
+        # growth are bracketed by an event pair on their stream; the elapsed times land in last_migrate_ms /
+        # last_fill_ms (the fill's when the caller next reads it: see fill_ms())
+        self.time_kernels = False
+        self.last_migrate_ms: Optional[float] = None
+        self.last_relocate_s: Optional[float] = None     # host time of the last relocation, its final wait included
+        self._fill_events: List[Tuple[torch.cuda.Event, torch.cuda.Event]] = []
+
+    def fill_ms(self) -> float:
+        """GPU time of the zero fills recorded since the last call (synchronises their events)."""
+        total = 0.0
+        for e0, e1 in self._fill_events:
+            e1.synchronize()
+            total += e0.elapsed_time(e1)
+        self._fill_events = []
+        return total
+
+    def _fill_zero(self, ptr: int, nbytes: int, stream: int) -> None:
+        timed = self.time_kernels
+        if timed:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+        _capi.check(_capi.lib().mkv_fill_zero(ptr, nbytes, stream))
+        if timed:
+            e1.record()
+            self._fill_events.append((e0, e1))
 
     # -- description ---------------------------------------------------------------
     @property
@@ -86,8 +116,8 @@ class ElasticKVPool:
         assert tuple(k_seg.shape) == (seg_blocks, *self.shape_tail) and k_seg.is_contiguous()
         assert tuple(v_seg.shape) == (seg_blocks, *self.shape_tail) and v_seg.is_contiguous()
         nbytes = seg_blocks * self.block_bytes
-        _capi.check(lib.mkv_fill_zero(k_seg.data_ptr(), nbytes, stream))
-        _capi.check(lib.mkv_fill_zero(v_seg.data_ptr(), nbytes, stream))
+        self._fill_zero(k_seg.data_ptr(), nbytes, stream)
+        self._fill_zero(v_seg.data_ptr(), nbytes, stream)
         self.k_cache_new.append(k_seg)
         self.v_cache_new.append(v_seg)
         self.kv_cache_new_block_size = seg_blocks
@@ -150,6 +180,7 @@ class ElasticKVPool:
         this returns no live block has an id >= ``new_num_blocks`` and the memory behind
         those ids is no longer read.  Raises ``PoolTooFullError`` (state untouched) when the
         live blocks do not fit below the cut; a failing launch raises ``MorphKVError``."""
+        t_start = time.perf_counter()
         _deferred.flush()
         bm = self.block_manager
         lib = _capi.lib()
@@ -165,13 +196,21 @@ class ElasticKVPool:
         if status != 0:
             raise PoolTooFullError(f"cannot shrink to {new_num_blocks} blocks: {moves} live blocks to move, "
                                f"{free_below} free below the cut")
+        events = None
         if moves:
             pool = self.descriptor()
+            if self.time_kernels:
+                events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                events[0].record()
             _capi.check(lib.mkv_pool_migrate(C.byref(pool), src.data_ptr(), dst.data_ptr(), moves, stream))
+            if events:
+                events[1].record()
             _capi.check(lib.mkv_bt_remap(bm.block_table.data_ptr(), bm.block_table.shape[1],
                                          bm.num_seq_allocated_blocks.data_ptr(),
                                          bm.num_seq_allocated_blocks.shape[0], remap.data_ptr(),
                                          bm.num_blocks, stream))
         # the memory above the cut must outlive the copy that reads it
         torch.cuda.current_stream().synchronize()
+        self.last_migrate_ms = events[0].elapsed_time(events[1]) if events else None
+        self.last_relocate_s = time.perf_counter() - t_start
         return src[:moves], dst[:moves]

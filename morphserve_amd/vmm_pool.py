@@ -128,6 +128,7 @@ class VmmKVPool(ElasticKVPool):
         self.block_manager = BlockManager("GPU", num_blocks, max_seqs_in_block_table, max_blocks_per_seq,
                                           block_size, device=device, reserve_blocks=max_blocks)
         self._result = torch.zeros(4, dtype=torch.int64, device=device)
+        self._init_timing()
         self._map(num_blocks)
         self._zero(0, num_blocks)
 
@@ -161,10 +162,10 @@ class VmmKVPool(ElasticKVPool):
                                        device=self.device)
 
     def _zero(self, first: int, count: int) -> None:
-        lib, stream = _capi.lib(), _capi.current_stream()
+        stream = _capi.current_stream()
         off, nbytes = first * self.block_bytes, count * self.block_bytes
-        _capi.check(lib.mkv_fill_zero(self._k_arena.base + off, nbytes, stream))
-        _capi.check(lib.mkv_fill_zero(self._v_arena.base + self._v_off + off, nbytes, stream))
+        self._fill_zero(self._k_arena.base + off, nbytes, stream)
+        self._fill_zero(self._v_arena.base + self._v_off + off, nbytes, stream)
 
     def descriptor(self) -> _capi.MkvPool:
         return _capi.make_pool(self.k_cache, self.v_cache)

@@ -74,12 +74,19 @@ class BlockManager:
         # given host lists (or re-read from the device by _host_counts after one that was not)
         self._host_n_alloc = np.zeros(max_seqs_in_block_table, dtype=np.int64)
         self._host_n_alloc_valid = True
+        # torch counts the in-place operations on a tensor: a change of that count means that code outside the
+        # manager wrote the device counts (a state loaded with copy_, an indexed assignment), and the host
+        # copy is re-read; the manager's own kernels write through the raw pointer and do not move it
+        self._host_n_alloc_version = self.num_seq_allocated_blocks._version
 
     # -- the host copy of the rows' block counts ------------------------------------------------------------
     def _host_counts(self) -> np.ndarray:
-        if not self._host_n_alloc_valid:          # a call without host lists changed the counts: one read back
+        version = self.num_seq_allocated_blocks._version
+        if not self._host_n_alloc_valid or version != self._host_n_alloc_version:
+            # a call without host lists, or code outside the manager, changed the counts: one read back
             self._host_n_alloc = self.num_seq_allocated_blocks.cpu().numpy().astype(np.int64)
             self._host_n_alloc_valid = True
+            self._host_n_alloc_version = version
         return self._host_n_alloc
 
     def invalidate_host_counts(self) -> None:

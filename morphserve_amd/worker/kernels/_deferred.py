@@ -47,6 +47,11 @@ class _State(threading.local):
 _state = _State()
 
 
+def pending() -> Optional[_Pending]:
+    """The calling thread's remembered append, if any."""
+    return _state.pending
+
+
 def enable_deferred_decode_append(on: bool) -> None:
     global ENABLED
     flush()

@@ -9,6 +9,13 @@ never leave the device -- the copy is one kernel reading both lists where the re
 does ``.tolist()`` twice and issues a memcpy pair per run of consecutive ids.
 ``use_kernel=False`` keeps the reference's route (host lists, memcpy runs) for pageable
 swap space.
+
+``cpu_tables="host"`` keeps the "CPU" block manager's tables in pinned host memory
+(``HostBlockManager``; the reference's live on the GPU, model.py:214-227): its side of a swap is then
+plain host work and its id list reaches the copy kernel through a pinned staging buffer.  Measured
+against the device-resident manager (``bench.py --workload eviction``) the two are equal within a
+percent -- a swap is bound by the PCIe copy, not by either manager -- so the device-resident one
+stays the default, as in the reference.
 """
 from __future__ import annotations
 
@@ -20,18 +27,27 @@ import torch
 from .. import _capi, swiftllm_c
 from ..elastic_pool import ElasticKVPool
 from .block_manager import BlockManager
+from .host_block_manager import HostBlockManager
 from .kernels import _deferred
 
 
 class KVSwapper:
     def __init__(self, pool: ElasticKVPool, num_cpu_blocks: int, cpu_block_manager: Optional[BlockManager] = None,
-                 pinned: bool = True):
+                 pinned: bool = True, cpu_tables: str = "device"):
+        if cpu_tables not in ("device", "host"):
+            raise ValueError('cpu_tables must be "device" or "host"')
         bm = pool.block_manager
         self.pool = pool
         self.gpu_block_manager = bm
-        self.cpu_block_manager = cpu_block_manager or BlockManager(
-            "CPU", num_cpu_blocks, bm.block_table.shape[0], bm.block_table.shape[1], bm.block_size,
-            device=str(pool.device))
+        if cpu_block_manager is not None:
+            self.cpu_block_manager = cpu_block_manager
+        elif cpu_tables == "host":
+            self.cpu_block_manager = HostBlockManager("CPU", num_cpu_blocks, bm.block_table.shape[0],
+                                                      bm.block_table.shape[1], bm.block_size)
+        else:
+            self.cpu_block_manager = BlockManager("CPU", num_cpu_blocks, bm.block_table.shape[0],
+                                                  bm.block_table.shape[1], bm.block_size, device=str(pool.device))
+        self._host_tables = isinstance(self.cpu_block_manager, HostBlockManager)
         shape = (num_cpu_blocks, *pool.shape_tail)
         self.k_swap = torch.zeros(shape, dtype=torch.float16, device="cpu", pin_memory=pinned)
         self.v_swap = torch.zeros(shape, dtype=torch.float16, device="cpu", pin_memory=pinned)
@@ -44,6 +60,25 @@ class KVSwapper:
         self._stage_dev = [torch.empty((2, rows), dtype=torch.int32, device=pool.device) for _ in range(2)]
         self._stage_done = [None, None]
         self._stage_turn = 0
+        if self._host_tables:                         # the host manager's id lists travel the same way
+            self._ids_host = [torch.empty(num_cpu_blocks, dtype=torch.int64, pin_memory=on_gpu) for _ in range(2)]
+            self._ids_dev = [torch.empty(num_cpu_blocks, dtype=torch.int64, device=pool.device) for _ in range(2)]
+            self._ids_done = [None, None]
+            self._ids_turn = 0
+
+    def _stage_ids(self, ids) -> torch.Tensor:
+        """A host id list as an int64 device tensor (asynchronous copy from pinned memory)."""
+        n = len(ids)
+        slot = self._ids_turn
+        self._ids_turn ^= 1
+        if self._ids_done[slot] is not None:
+            self._ids_done[slot].synchronize()
+        self._ids_host[slot].numpy()[:n] = ids
+        self._ids_dev[slot][:n].copy_(self._ids_host[slot][:n], non_blocking=True)
+        if self._ids_dev[slot].is_cuda:
+            self._ids_done[slot] = torch.cuda.Event()
+            self._ids_done[slot].record()
+        return self._ids_dev[slot][:n]
 
     def _stage(self, ids_host, lens_host):
         """Device views of the two lists, copied asynchronously from pinned memory on the current stream."""
@@ -75,11 +110,24 @@ class KVSwapper:
         # (model.py:481-489 reads them back three times)
         lens_host = src_mgr.host_num_allocated_blocks(ids_host) * self.gpu_block_manager.block_size
         seq_ids, seq_lengths = self._stage(ids_host, lens_host)
-        src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids, seq_ids_host=ids_host)    # int32, sequence-major
-        dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths, seq_ids_host=ids_host,
-                                                   target_lens_host=lens_host)             # int64, lowest free ids
-        n = int(src_ids.numel())
-        assert int(dst_ids.numel()) == n
+        src_host = dst_host = None
+        if self._host_tables and is_swap_in:           # the host manager gives, the device manager takes
+            src_host = src_mgr.gather_allocated_blocks_and_free(ids_host)
+            dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths, seq_ids_host=ids_host,
+                                                       target_lens_host=lens_host)
+            src_ids = self._stage_ids(src_host) if use_kernel else None
+            n = len(src_host)
+        elif self._host_tables:
+            src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids, seq_ids_host=ids_host)
+            dst_host = dst_mgr.allocate_blocks_for_seqs(ids_host, lens_host)
+            dst_ids = self._stage_ids(dst_host) if use_kernel else None
+            n = len(dst_host)
+        else:
+            src_ids = src_mgr.gather_allocated_blocks_and_free(seq_ids, seq_ids_host=ids_host)    # int32, sequence-major
+            dst_ids = dst_mgr.allocate_blocks_for_seqs(seq_ids, seq_lengths, seq_ids_host=ids_host,
+                                                       target_lens_host=lens_host)             # int64, lowest free ids
+            n = int(src_ids.numel())
+            assert int(dst_ids.numel()) == n
         self.block_swap += n
         if n == 0:
             return 0
@@ -96,7 +144,8 @@ class KVSwapper:
         else:
             desc = self.pool.descriptor()
             cnt = C.c_int64(0)
-            src_l, dst_l = src_ids.tolist(), dst_ids.tolist()
+            src_l = src_host.tolist() if src_host is not None else src_ids.tolist()
+            dst_l = dst_host.tolist() if dst_host is not None else dst_ids.tolist()
             _capi.check(_capi.lib().mkv_swap_blocks(
                 swiftllm_c._ids(src_l), swiftllm_c._ids(dst_l), n, 1 if is_swap_in else 0, C.byref(desc),
                 self.k_swap.data_ptr(), self.v_swap.data_ptr(), C.byref(cnt), _capi.current_stream()))
@@ -115,4 +164,7 @@ class KVSwapper:
         ids_host = list(seq_ids_list)
         seq_ids, _ = self._stage(ids_host, [0] * len(ids_host))
         self.gpu_block_manager.free_blocks_for_seqs(seq_ids, seq_ids_host=ids_host)
-        self.cpu_block_manager.free_blocks_for_seqs(seq_ids, seq_ids_host=ids_host)
+        if self._host_tables:
+            self.cpu_block_manager.free_blocks_for_seqs(ids_host)
+        else:
+            self.cpu_block_manager.free_blocks_for_seqs(seq_ids, seq_ids_host=ids_host)

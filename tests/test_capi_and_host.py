@@ -299,3 +299,55 @@ def test_step_state_builder_matches_the_field_by_field_builder():
         b.build([4000, 200], [0, 1], [])
     with pytest.raises(ValueError):
         b.build([], [0, 1], [5])
+
+
+def test_decode_order_cache_is_tied_to_the_capture_it_was_made_in(monkeypatch):
+    """The balanced row order is computed by a launch and kept on the infer state.  A launch that was only
+    RECORDED into a graph has written nothing yet, so an entry made during a stream capture must serve that
+    capture alone: an eager call (the capture may have been abandoned) and any other capture compute their own.
+    Host logic only: the library, the stream and the events are stand-ins."""
+    import torch
+
+    from morphserve_amd.worker.kernels import paged_attn as PA
+    launches = []
+
+    class Lib:
+        def mkv_decode_order(self, lens_ptr, n, hkv, order_ptr, stream):
+            launches.append(order_ptr)
+            return 0
+
+    class Stream:
+        cuda_stream = 7
+
+        def wait_event(self, event):
+            pass
+
+    class Event:
+        def record(self, stream):
+            pass
+
+    capture = {"id": None}
+    monkeypatch.setattr(PA._capi, "lib", lambda: Lib())
+    monkeypatch.setattr(PA._capi, "capture_id", lambda stream: capture["id"])
+    monkeypatch.setattr(PA.torch.cuda, "current_stream", lambda: Stream())
+    monkeypatch.setattr(PA.torch.cuda, "Event", Event)
+    monkeypatch.setattr(PA, "BALANCED_ORDER", True)
+
+    class State:
+        pass
+    state, lens = State(), torch.zeros(8, dtype=torch.int32)
+    eager = PA._decode_order(state, lens, 8, 2, 1)
+    assert len(launches) == 1 and PA._decode_order(state, lens, 8, 2, 1) is eager and len(launches) == 1
+    capture["id"] = 5                                   # a capture begins: the eager entry is not carried into it
+    in_graph = PA._decode_order(state, lens, 8, 2, 1)
+    assert in_graph is not eager and len(launches) == 2
+    assert PA._decode_order(state, lens, 8, 2, 1) is in_graph and len(launches) == 2      # the other layers of the capture
+    capture["id"] = None                                # eager again (graph not replayed, or abandoned)
+    after = PA._decode_order(state, lens, 8, 2, 1)
+    assert after is not in_graph and len(launches) == 3 and launches[2] == after.data_ptr()
+    capture["id"] = 6                                   # another capture
+    assert PA._decode_order(state, lens, 8, 2, 1) is not after and len(launches) == 4
+    # nothing to balance: one row, a split batch, or the switch off
+    assert PA._decode_order(state, lens[:1], 1, 2, 1) is None and PA._decode_order(state, lens, 8, 2, 3) is None
+    monkeypatch.setattr(PA, "BALANCED_ORDER", False)
+    assert PA._decode_order(state, lens, 8, 2, 1) is None and len(launches) == 4

@@ -18,7 +18,7 @@ def deferral():
     M.enable_deferred_decode_append(True)
     yield
     M.enable_deferred_decode_append(False)
-    assert _deferred._pending is None
+    assert _deferred.pending() is None
 
 
 def _setup(cuda, seed, Hq, Hkv, p_lens, d_lens, L=3):
@@ -50,7 +50,7 @@ def test_deferred_rows_are_appended_by_the_attention_launch(cuda, deferral, Hq, 
     before_k = bits(kc).copy()
     M.store_kvcache(kg, vg, kc, vc, [], [], bt, model, engine, st, layer)
     torch.cuda.synchronize()
-    assert _deferred._pending is not None
+    assert _deferred.pending() is not None
     # only the prefill rows have been written so far
     ref = make_case(41, 3, Hq, Hkv, list(p_lens) + list(d_lens), num_blocks=case.num_blocks, fill="all")
     if p_lens:
@@ -64,7 +64,7 @@ def test_deferred_rows_are_appended_by_the_attention_launch(cuda, deferral, Hq, 
     o = torch.full((n, Hq * 128), float("nan"), dtype=torch.float16, device=cuda)
     M.paged_attention(torch.from_numpy(q).to(cuda), kc, vc, [], [], bt, model, engine, st, layer, o)
     torch.cuda.synchronize()
-    assert _deferred._pending is None
+    assert _deferred.pending() is None
     _oracle_store(case, k, v, p_lens, d_lens, T, layer)
     assert np.array_equal(bits(kc), bits(case.k_pool)) and np.array_equal(bits(vc), bits(case.v_pool))
     want = R.paged_attention(q, case.arena, case.lay, case.block_table, case.seq_ids[len(p_lens):],
@@ -86,7 +86,7 @@ def test_every_other_route_issues_the_pending_append(cuda, deferral):
     # (3) an attention call for a DIFFERENT layer issues it, then attends without appending
     M.paged_attention(qg, kc, vc, [], [], bt, model, engine, st, 0, o)
     torch.cuda.synchronize()
-    assert _deferred._pending is None
+    assert _deferred.pending() is None
     for layer in range(3):
         R.append_decode(case.arena, case.lay, k, v, case.block_table, case.seq_ids, np.asarray(d_lens), layer)
     assert np.array_equal(bits(kc), bits(case.k_pool)) and np.array_equal(bits(vc), bits(case.v_pool))
@@ -95,7 +95,7 @@ def test_every_other_route_issues_the_pending_append(cuda, deferral):
     # (4) switching the deferral off issues what is pending
     M.store_kvcache(kg, vg, kc, vc, [], [], bt, model, engine, st, 1)
     M.enable_deferred_decode_append(False)
-    assert _deferred._pending is None
+    assert _deferred.pending() is None
     M.enable_deferred_decode_append(True)
 
 

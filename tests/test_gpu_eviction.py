@@ -20,12 +20,13 @@ def _oracle_swap(arena, lay, src_bm, dst_bm, ks, vs, seq_ids, is_swap_in):
     return len(src)
 
 
+@pytest.mark.parametrize("cpu_tables", ["device", "host"])
 @pytest.mark.parametrize("use_kernel,pinned", [(True, True), (False, True), (False, False)])
-def test_swap_out_and_back_matches_the_oracle(cuda, use_kernel, pinned):
+def test_swap_out_and_back_matches_the_oracle(cuda, use_kernel, pinned, cpu_tables):
     org, S, nseg = 16, 8, 3
     pool, ob, arena, lay = pool_case(cuda, 5, org, S, nseg, 0.5)
     n_cpu = 40
-    sw = KVSwapper(pool, n_cpu, pinned=pinned)
+    sw = KVSwapper(pool, n_cpu, pinned=pinned, cpu_tables=cpu_tables)
     assert sw.k_swap.is_pinned() == pinned
     ocpu = R.BlockManagerOracle("CPU", n_cpu, 24, org + nseg * S, 16)
     ks = np.zeros(sw.k_swap.shape, dtype=np.float16)
