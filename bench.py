@@ -1361,6 +1361,13 @@ def bench_allocator(args):
         cur = np.zeros(64, dtype=np.int64)
         times = {}
         for mode in ("host lists", "device read"):
+            for _ in range(3):                             # warm-up: code objects, torch's allocator, the host copy
+                cur += 16
+                tgt = torch.from_numpy(cur.astype(np.int32)).to(dev)
+                if mode == "host lists":
+                    bm.allocate_blocks_for_seqs(ids, tgt, seq_ids_host=ids_h, target_lens_host=cur)
+                else:
+                    bm.allocate_blocks_for_seqs(ids, tgt)
             reps = max(args.steps, 20)
             host_s = 0.0
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

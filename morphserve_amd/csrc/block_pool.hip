@@ -6,6 +6,8 @@
 // trips between the steps.
 #include "common.h"
 
+#include <algorithm>
+
 namespace mkv {
 
 static constexpr int kScanThreads = 1024;
@@ -107,12 +109,43 @@ __device__ int64_t count_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8
     return seen;
 }
 
+// Position (0 .. 63) of the r-th set bit of `bits` (r counted from 0, r < popcount).
+__device__ __forceinline__ int select64(uint64_t bits, int r) {
+    uint32_t w = (uint32_t)bits;
+    int off = 0;
+    int c = __popc(w);
+    if (r >= c) {
+        r -= c;
+        w = (uint32_t)(bits >> 32);
+        off = 32;
+    }
+#pragma unroll
+    for (int shift = 16; shift >= 1; shift >>= 1) {
+        c = __popc(w & ((1u << shift) - 1u));
+        if (r >= c) {
+            r -= c;
+            w >>= shift;
+            off += shift;
+        }
+    }
+    return off;
+}
+
 // Writes the first `n` positions of map[lo, hi) whose byte equals `want`, ascending, to out[0..n)
 // (and the first kIdCache of them to `cache`, when given) WITHOUT touching the map; returns how many
 // were found, which is below n only when the range holds fewer.  `first_bits` / `have_first`: the
 // mask of the first tile when the caller has requested it early.  All threads must call it.
+//
+// Two ways to turn a tile's masks into positions.  When a tile contributes many positions every thread
+// walks its own mask (64 bytes, up to 64 stores).  When it contributes few -- the usual allocation: a
+// handful of blocks out of a map that is mostly free -- those few would all sit in the first threads'
+// masks and one lane would walk them alone; then thread p finds the p-th position itself, by a binary
+// search over the threads' running counts and a select inside the mask it lands in, and the stores are
+// coalesced.
 __device__ int64_t collect_bytes(const uint8_t* map, int64_t lo, int64_t hi, uint8_t want, int64_t n,
                                  int64_t* out, int32_t* cache, int32_t* sm, uint64_t first_bits, bool have_first) {
+    __shared__ int32_t s_pref[kScanThreads];
+    __shared__ uint64_t s_mask[kScanThreads];
     int64_t base = 0;
     bool first = true;
     for (int64_t t0 = aligned_start(map, lo); t0 < hi && base < n; t0 += kTileBytes) {
@@ -121,13 +154,33 @@ __device__ int64_t collect_bytes(const uint8_t* map, int64_t lo, int64_t hi, uin
         first = false;
         const int32_t c = __popcll(bits);
         int32_t tot;
-        int64_t pos = base + block_excl_scan<int32_t>(c, &tot, sm);
-        while (bits != 0ull && pos < n) {
-            const int k = __builtin_ctzll(bits);
-            bits &= bits - 1;
-            out[pos] = b0 + k;
-            if (cache != nullptr && pos < kIdCache) cache[pos] = (int32_t)(b0 + k);
-            ++pos;
+        const int32_t excl = block_excl_scan<int32_t>(c, &tot, sm);
+        const int64_t take = min((int64_t)tot, n - base);           // positions this tile contributes
+        if (take <= 2 * kScanThreads) {
+            s_pref[threadIdx.x] = excl;
+            s_mask[threadIdx.x] = bits;
+            __syncthreads();
+            for (int64_t p = threadIdx.x; p < take; p += kScanThreads) {
+                int lo_t = 0, hi_t = kScanThreads - 1;               // last thread whose running count is <= p
+                while (lo_t < hi_t) {
+                    const int mid = (lo_t + hi_t + 1) >> 1;
+                    if (s_pref[mid] <= (int32_t)p) lo_t = mid; else hi_t = mid - 1;
+                }
+                const int k = select64(s_mask[lo_t], (int)p - s_pref[lo_t]);
+                const int64_t id = t0 + (int64_t)lo_t * kBytesPerThread + k;
+                out[base + p] = id;
+                if (cache != nullptr && base + p < kIdCache) cache[base + p] = (int32_t)id;
+            }
+            __syncthreads();                                         // the arrays are reused by the next tile
+        } else {
+            int64_t pos = base + excl;
+            while (bits != 0ull && pos < n) {
+                const int k = __builtin_ctzll(bits);
+                bits &= bits - 1;
+                out[pos] = b0 + k;
+                if (cache != nullptr && pos < kIdCache) cache[pos] = (int32_t)(b0 + k);
+                ++pos;
+            }
         }
         base += tot;
     }
@@ -155,8 +208,10 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
                                              num_blocks, 1);
     __syncthreads();
 
-    // pass 1: total need, precondition need_i >= 0 and room in the table row
-    int64_t my_need = 0;
+    // pass 1: total need, precondition need_i >= 0 and room in the table row.  A thread keeps the row it
+    // reads first (row tid: the whole batch when it has at most 1024 rows), so that handing the ids out
+    // does not have to fetch the row's sequence id and count a second time.
+    int64_t my_need = 0, r_seq = 0, r_have = 0, r_need = 0;
     for (int i = tid; i < batch; i += kScanThreads) {
         const int64_t target = ((int64_t)target_lens[i] + block_size - 1) / block_size;
         const int64_t seq = seq_ids[i];
@@ -166,9 +221,11 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
         if (target > max_blocks_per_seq) atomicMax(&s_bad, 2);   // would not fit the table row
         else if (need < 0) atomicMax(&s_bad, 1);
         my_need += need;
+        if (i == tid) { r_seq = seq; r_have = have; r_need = need; }
     }
     int64_t total;
-    block_excl_scan<int64_t>(my_need, &total, sm);
+    // with at most one row per thread this is also every row's first position in the list of new ids
+    const int64_t r_start = block_excl_scan<int64_t>(my_need, &total, sm);
     __syncthreads();
     if (s_bad) {
         if (tid == 0) { result[0] = total; result[1] = (s_bad == 2) ? MKV_EINVAL : MKV_ELOGIC; result[2] = 0; }
@@ -198,13 +255,15 @@ __global__ __launch_bounds__(kScanThreads) void bm_allocate_kernel(
     for (int i0 = 0; i0 < batch; i0 += kScanThreads) {
         const int i = i0 + tid;
         int64_t need = 0, have = 0, seq = 0;
-        if (i < batch) {
+        if (i0 == 0) {                                       // the rows remembered from pass 1
+            if (i < batch) { seq = r_seq; have = r_have; need = r_need; }
+        } else if (i < batch) {
             seq = seq_ids[i];
             have = n_alloc[seq];
             need = ((int64_t)target_lens[i] + block_size - 1) / block_size - have;
         }
-        int64_t tot;
-        const int64_t start = base + block_excl_scan<int64_t>(need, &tot, sm);
+        int64_t tot = total, start = r_start;
+        if (batch > kScanThreads) start = base + block_excl_scan<int64_t>(need, &tot, sm);
         if (i < batch && need > 0) {
             int32_t* dst = block_table + seq * max_blocks_per_seq + have;
             for (int64_t x = 0; x < need; ++x) {
@@ -387,13 +446,161 @@ __global__ __launch_bounds__(kScanThreads) void pool_plan_shrink_kernel(
     }
     __threadfence_block();
     __syncthreads();
-    for (int64_t k = tid; k < moves; k += kScanThreads) {
+    // four moves per thread and round, every load ahead of the stores (the lists were written by other
+    // threads: each round is a trip to the L2)
+    for (int64_t k0 = tid; k0 < moves; k0 += 4 * kScanThreads) {
+        int64_t s_id[4], d_id[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t k = k0 + (int64_t)u * kScanThreads;
+            s_id[u] = k < moves ? src[k] : -1;
+            d_id[u] = k < moves ? dst[k] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (s_id[u] >= 0) {
+                is_free[s_id[u]] = 1;
+                is_free[d_id[u]] = 0;
+                remap[s_id[u]] = (int32_t)d_id[u];
+            }
+    }
+    if (tid == 0) { result[0] = moves; result[1] = MKV_OK; result[2] = free_below; }
+}
+
+// ---- shrink planning over many workgroups (large maps) -----------------------------------
+// One workgroup cannot enumerate ten thousand positions of a 100 k map in much under 30 us: the
+// enumeration and its scattered stores are one CU's work.  For large maps the plan is three launches
+// of one workgroup per 4096 map bytes:
+//   count  every tile counts its free bytes below the cut and its live bytes above it, and writes
+//          the identity into its part of remap (the counts travel in remap[0 .. 2T), which no move
+//          ever writes: moved ids are >= new_n >= 2T, the host checks);
+//   place  every workgroup sums the counts of the tiles before it (T is small), decides whether the
+//          plan fits (all workgroups see the same totals) and, if it does, writes its tile's live ids
+//          above the cut into src and its free ids below the cut, up to the number needed, into dst;
+//   apply  restores the identity in remap[0 .. 2T) and applies the moves to the map and to remap.
+// Nothing but scratch (src, dst, remap) is written unless the plan fits.
+static constexpr int kPlanThreads = 256;
+static constexpr int kPlanTileBytes = kPlanThreads * 16;
+
+__device__ __forceinline__ uint32_t plan_mask16(const uint8_t* map, int64_t b0, int64_t lo, int64_t hi, uint8_t want) {
+    if (b0 + 16 <= lo || b0 >= hi) return 0u;
+    uint32_t nz = 0u, in = 0xffffu;
+    if (b0 >= lo && b0 + 16 <= hi && (((uintptr_t)(map + b0)) & 15u) == 0) {
+        nz = nonzero_mask16(*(const uint4*)(map + b0));
+    } else {
+        in = 0u;
+        for (int k = 0; k < 16; ++k) {
+            const int64_t b = b0 + k;
+            if (b >= lo && b < hi) {
+                in |= 1u << k;
+                if (map[b] != 0) nz |= 1u << k;
+            }
+        }
+    }
+    return (want != 0 ? nz : ~nz) & in;
+}
+
+// sum over the 256 threads of a plan workgroup; all threads call it
+__device__ __forceinline__ int32_t plan_block_sum(int32_t v, int32_t* sm /* [4] */) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return sm[0] + sm[1] + sm[2] + sm[3];
+}
+
+__global__ __launch_bounds__(kPlanThreads) void plan_count_kernel(const uint8_t* __restrict__ is_free, int64_t num_blocks,
+                                                                  int64_t new_n, int32_t* __restrict__ remap, int32_t tiles) {
+    __shared__ int32_t sm[4];
+    const int64_t b0 = (int64_t)blockIdx.x * kPlanTileBytes + (int64_t)threadIdx.x * 16;
+    const int32_t free_below = __popc(plan_mask16(is_free, b0, 0, new_n, 1));
+    const int32_t live_above = __popc(plan_mask16(is_free, b0, new_n, num_blocks, 0));
+    for (int k = 0; k < 16; ++k) {
+        const int64_t b = b0 + k;
+        if (b < num_blocks && b >= 2 * (int64_t)tiles) remap[b] = (int32_t)b;
+    }
+    const int32_t f = plan_block_sum(free_below, sm);
+    const int32_t l = plan_block_sum(live_above, sm);
+    if (threadIdx.x == 0) {
+        remap[2 * blockIdx.x] = f;
+        remap[2 * blockIdx.x + 1] = l;
+    }
+}
+
+__global__ __launch_bounds__(kPlanThreads) void plan_place_kernel(const uint8_t* __restrict__ is_free, int64_t num_blocks,
+                                                                  int64_t new_n, int64_t* __restrict__ src,
+                                                                  int64_t* __restrict__ dst, int64_t cap,
+                                                                  const int32_t* __restrict__ remap, int32_t tiles,
+                                                                  int64_t* __restrict__ result) {
+    __shared__ int32_t sm[4];
+    __shared__ int32_t s_scan[kPlanThreads / 64 + 1];
+    const int tid = threadIdx.x;
+    // totals and this tile's offsets from the per-tile counts
+    int32_t f_before = 0, l_before = 0, f_all = 0, l_all = 0;
+    for (int t = tid; t < tiles; t += kPlanThreads) {
+        const int32_t f = remap[2 * t], l = remap[2 * t + 1];
+        f_all += f;
+        l_all += l;
+        if (t < (int)blockIdx.x) { f_before += f; l_before += l; }
+    }
+    f_before = plan_block_sum(f_before, sm);
+    l_before = plan_block_sum(l_before, sm);
+    f_all = plan_block_sum(f_all, sm);
+    l_all = plan_block_sum(l_all, sm);
+    const int64_t moves = l_all;
+    const bool fits = moves <= cap && (int64_t)f_all >= moves;
+    if (blockIdx.x == 0 && tid == 0) {
+        result[0] = moves;
+        result[1] = fits ? MKV_OK : MKV_ENOSPC;
+        result[2] = f_all < moves ? f_all : (fits ? moves : f_all);
+    }
+    if (!fits) return;
+    const int64_t b0 = (int64_t)blockIdx.x * kPlanTileBytes + (int64_t)tid * 16;
+    const int lane = tid & 63, wave = tid >> 6;
+    // two ordered compactions of this tile: live above the cut -> src, free below the cut -> dst
+    for (int which = 0; which < 2; ++which) {
+        const uint32_t bits = which == 0 ? plan_mask16(is_free, b0, new_n, num_blocks, 0)
+                                         : plan_mask16(is_free, b0, 0, new_n, 1);
+        const int32_t c = __popc(bits);
+        int32_t inc = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int32_t t = __shfl_up(inc, d);
+            if (lane >= d) inc += t;
+        }
+        __syncthreads();
+        if (lane == 63) s_scan[wave] = inc;
+        __syncthreads();
+        int32_t wave_off = 0;
+        for (int w = 0; w < wave; ++w) wave_off += s_scan[w];
+        int64_t pos = (int64_t)(which == 0 ? l_before : f_before) + wave_off + inc - c;
+        int64_t* out = which == 0 ? src : dst;
+        if (c != 0 && pos < moves) {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                if ((bits >> k) & 1u) {
+                    if (pos < moves) out[pos] = b0 + k;
+                    ++pos;
+                }
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kPlanThreads) void plan_apply_kernel(uint8_t* __restrict__ is_free, const int64_t* __restrict__ src,
+                                                                  const int64_t* __restrict__ dst, int32_t* __restrict__ remap,
+                                                                  int32_t tiles, const int64_t* __restrict__ result) {
+    if (blockIdx.x == 0)                              // the counts have been read: their slots become identity again
+        for (int b = threadIdx.x; b < 2 * tiles; b += kPlanThreads) remap[b] = b;
+    if (result[1] != MKV_OK) return;
+    const int64_t moves = result[0];
+    for (int64_t k = (int64_t)blockIdx.x * kPlanThreads + threadIdx.x; k < moves; k += (int64_t)gridDim.x * kPlanThreads) {
         const int64_t s_id = src[k], d_id = dst[k];
         is_free[s_id] = 1;
         is_free[d_id] = 0;
         remap[s_id] = (int32_t)d_id;
     }
-    if (tid == 0) { result[0] = moves; result[1] = MKV_OK; result[2] = free_below; }
 }
 
 __global__ __launch_bounds__(256) void bt_remap_kernel(int32_t* __restrict__ block_table,
@@ -520,9 +727,22 @@ int mkv_pool_plan_shrink(uint8_t* is_block_free, int64_t num_blocks, int64_t new
                 (long long)num_blocks);
     MKV_REQUIRE(num_blocks <= INT32_MAX, "block ids must fit int32");
     MKV_REQUIRE((src && dst) || cap == 0, "src/dst are NULL");
-    hipLaunchKernelGGL(mkv::pool_plan_shrink_kernel, dim3(1), dim3(mkv::kScanThreads), 0,
-                       (hipStream_t)stream, is_block_free, num_blocks, new_num_blocks, src, dst,
-                       cap, remap, result);
+    // large maps: one workgroup per 4096 bytes in three launches (the per-tile counts travel in the first
+    // 2 * tiles entries of remap, which must lie below the cut); small ones: one workgroup does it all
+    const int64_t tiles = (num_blocks + mkv::kPlanTileBytes - 1) / mkv::kPlanTileBytes;
+    hipStream_t s = (hipStream_t)stream;
+    if (num_blocks >= 32768 && 2 * tiles <= new_num_blocks && tiles <= 65535 && cap > 0) {
+        hipLaunchKernelGGL(mkv::plan_count_kernel, dim3((unsigned)tiles), dim3(mkv::kPlanThreads), 0, s, is_block_free,
+                           num_blocks, new_num_blocks, remap, (int32_t)tiles);
+        hipLaunchKernelGGL(mkv::plan_place_kernel, dim3((unsigned)tiles), dim3(mkv::kPlanThreads), 0, s, is_block_free,
+                           num_blocks, new_num_blocks, src, dst, cap, remap, (int32_t)tiles, result);
+        const unsigned apply_grid = (unsigned)std::min<int64_t>(tiles, 2 * (int64_t)mkv::num_cus());
+        hipLaunchKernelGGL(mkv::plan_apply_kernel, dim3(apply_grid), dim3(mkv::kPlanThreads), 0, s, is_block_free, src, dst,
+                           remap, (int32_t)tiles, result);
+    } else {
+        hipLaunchKernelGGL(mkv::pool_plan_shrink_kernel, dim3(1), dim3(mkv::kScanThreads), 0, s, is_block_free, num_blocks,
+                           new_num_blocks, src, dst, cap, remap, result);
+    }
     MKV_HIP(hipGetLastError());
     return MKV_OK;
 }
