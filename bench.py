@@ -129,24 +129,33 @@ def decode_bytes_per_layer(lens, n, hq, hkv, d, b):
 
 
 def auto_chunk_blocks(num_blocks, bytes_per_block_and_tensor):
-    """The largest divisor of num_blocks whose chunk stays at or under 1 GiB per tensor."""
+    """Blocks per chunk for a pool of num_blocks: the largest count whose chunk is a multiple of 2 MiB and at
+    most 1 GiB per tensor, a divisor of num_blocks when one exists that gives chunks of 256 MiB and more (what
+    placement by memory groups needs), else the largest such count (the pool then maps whole chunks past
+    num_blocks)."""
     target = max(1, (1 << 30) // bytes_per_block_and_tensor)
-    for c in range(min(target, num_blocks), 0, -1):
-        if num_blocks % c == 0:
+    aligned = [c for c in range(min(target, num_blocks), 0, -1) if (c * bytes_per_block_and_tensor) % (2 << 20) == 0]
+    if not aligned:
+        return 1
+    for c in aligned:
+        if num_blocks % c == 0 and c * bytes_per_block_and_tensor >= (256 << 20):
             return c
-    return 1
+    return aligned[0]
 
 
 def make_pool(args, num_blocks, max_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq):
-    """The KV pool of a workload by --pool-backing / --placement; (pool, description)."""
+    """The KV pool of a workload by --pool-backing / --placement; (pool, description).  A virtual-memory pool
+    holds whole chunks: its block counts are the workload's rounded up to the chunk."""
     from morphserve_amd import ElasticKVPool, VmmKVPool
     if args.pool_backing == "vmm":
         per_tensor = L * HKV * B * D * 2
         chunk = args.vmm_chunk_blocks or auto_chunk_blocks(int(np.gcd(num_blocks, max_blocks)), per_tensor)
+        asked = num_blocks
+        num_blocks, max_blocks = -(-num_blocks // chunk) * chunk, -(-max_blocks // chunk) * chunk
         pool = VmmKVPool(num_blocks, max_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, chunk_blocks=chunk,
                          placement=args.placement, v_stagger_bytes=args.v_stagger_bytes)
         what = (f"VmmKVPool, chunks of {chunk} blocks ({chunk * per_tensor / 2**20:.0f} MiB per tensor), placement "
-                f"{args.placement}")
+                f"{args.placement}" + (f", {num_blocks} blocks mapped for the {asked} used" if num_blocks != asked else ""))
     else:
         pool = ElasticKVPool(num_blocks, L, HKV, B, D, max_seqs, max_blocks_per_seq, reserve_blocks=max_blocks)
         what = "ElasticKVPool: two torch allocations, growth by segments"
@@ -1017,7 +1026,7 @@ def bench_serving(args):
         t += rng.gamma(0.5, 10.0)
         arrival_step.append(int(t))
     next_arrival = 0
-    spent = {"schedule": 0.0, "allocate": 0.0, "kernels": 0.0, "free": 0.0}
+    spent = {"schedule": 0.0, "allocate": 0.0, "allocate_call_host": 0.0, "kernels": 0.0, "free": 0.0}
     counts = {"prefill_steps": 0, "decode_steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "finished": 0,
               "allocate_calls": 0, "blocks_allocated": 0, "max_running": 0}
 
@@ -1042,9 +1051,15 @@ def bench_serving(args):
         prefill = batch is not sched.running_q
         ids = [r.request_id for r in reqs]
         lens = [r.prompt_len + r.output_len for r in reqs]
-        new_ids = bm.allocate_blocks_for_seqs(dev_i32(ids), dev_i32(lens))
+        ids_t, lens_t = dev_i32(ids), dev_i32(lens)
+        t1a = time.perf_counter()
+        # the lists the scheduler already holds go along: every check and the size of the result come from the
+        # manager's host copy of its counters, nothing is read back from the device
+        new_ids = bm.allocate_blocks_for_seqs(ids_t, lens_t, seq_ids_host=ids, target_lens_host=lens)
+        t1b = time.perf_counter()
         torch.cuda.synchronize()
         t2 = time.perf_counter()
+        spent["allocate_call_host"] += t1b - t1a
         if prefill:
             p_lens, d_lens = [r.prompt_len for r in reqs], []
             positions = np.concatenate([np.arange(n) for n in p_lens])
@@ -1069,7 +1084,7 @@ def bench_serving(args):
             r.output_len += 1
         done = [r.request_id for r in reqs if r.is_finished()]
         if done:
-            bm.free_blocks_for_seqs(dev_i32(done))
+            bm.free_blocks_for_seqs(dev_i32(done), seq_ids_host=done)
             torch.cuda.synchronize()
         sched.on_batch_finish(reqs)
         t4 = time.perf_counter()
@@ -1105,7 +1120,8 @@ def bench_serving(args):
         **counts,
         "share_of_wall": {kk: round(vv / wall, 4) for kk, vv in spent.items()},
         "avg_ms": {"schedule": round(spent["schedule"] * 1e3 / n_steps, 4),
-                   "allocate_call": round(spent["allocate"] * 1e3 / max(counts["allocate_calls"], 1), 4),
+                   "allocate_call_host": round(spent["allocate_call_host"] * 1e3 / max(counts["allocate_calls"], 1), 4),
+                   "allocate_incl_input_copy_and_sync": round(spent["allocate"] * 1e3 / max(counts["allocate_calls"], 1), 4),
                    "kernels_per_step": round(spent["kernels"] * 1e3 / max(steps_run, 1), 4),
                    "free_and_bookkeeping": round(spent["free"] * 1e3 / max(steps_run, 1), 4)},
         "roofline": None,

@@ -342,7 +342,8 @@ int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes);
  * while it does).  Where an arena can still grow it also keeps one spare chunk of its group as the
  * reference for later calls (held until mkv_arena_destroy); a later call creates exactly the chunks
  * it needs, measures them against those references and gives each arena the ones of its own group
- * first.  Chunks under 256 MiB cannot be measured: plain growth.
+ * first.  Chunks under 256 MiB cannot be measured, and chunks that are no multiple of 2 MiB cannot be
+ * staged for the measurement: plain growth for both.
  * Host call; it synchronises `stream`, on which the measurement kernels run; the new memory holds
  * whatever the measurement left (the caller clears it, as after mkv_arena_resize).  MKV_ENOSPC when
  * the device has no memory left (nothing changed).  `info` (may be NULL) reports what was found. */

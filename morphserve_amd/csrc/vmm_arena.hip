@@ -14,7 +14,6 @@
 // never an absolute rate, so a device without such groups simply yields one group and the plain order.
 #include "common.h"
 
-#include <stdlib.h>
 #include <algorithm>
 #include <chrono>
 #include <vector>
@@ -52,7 +51,7 @@ static int arena_map_one(mkv_arena* a) {
     }
     if (e != hipSuccess) {
         (void)hipMemRelease(h);
-        MKV_HIP(e);
+        return ::mkv::hip_fail(e, "hipMemMap / hipMemSetAccess of a fresh chunk at the end of the arena");
     }
     a->chunks.push_back(h);
     return MKV_OK;
@@ -68,7 +67,7 @@ static int arena_map_handle(mkv_arena* a, hipMemGenericAllocationHandle_t h) {
     hipError_t e = hipMemSetAccess(at, a->chunk, &acc, 1);
     if (e != hipSuccess) {
         (void)hipMemUnmap(at, a->chunk);
-        MKV_HIP(e);
+        return ::mkv::hip_fail(e, "hipMemMap / hipMemSetAccess of a handed-over chunk at the end of the arena");
     }
     a->chunks.push_back(h);
     return MKV_OK;
@@ -270,14 +269,18 @@ struct PairGrow {
                 break;                                      // out of device memory: work with what there is
             }
             char* at = (char*)win + i * chunk;
+            const char* what = "hipMemMap";
             hipError_t e = hipMemMap(at, chunk, 0, h, 0);
             if (e == hipSuccess) {
+                what = "hipMemSetAccess";
                 e = hipMemSetAccess(at, chunk, &acc, 1);
                 if (e != hipSuccess) (void)hipMemUnmap(at, chunk);
             }
             if (e != hipSuccess) {
                 (void)hipMemRelease(h);
-                MKV_HIP(e);
+                set_error("HIP error %d (%s) in %s of candidate %zu of %zu in the staging window (chunks of %llu bytes)",
+                          (int)e, hipGetErrorString(e), what, i, n, (unsigned long long)chunk);
+                return MKV_EHIP;
             }
             cand.push_back({h, at, -1, false});
             ++*got;
@@ -335,7 +338,7 @@ static int map_ref(mkv_arena* a, hipMemGenericAllocationHandle_t h) {
     hipError_t e = hipMemSetAccess(a->ref_va, a->chunk, &acc, 1);
     if (e != hipSuccess) {
         (void)hipMemUnmap(a->ref_va, a->chunk);
-        MKV_HIP(e);
+        return ::mkv::hip_fail(e, "hipMemMap / hipMemSetAccess of the reference chunk");
     }
     a->ref = h;
     a->has_ref = true;
@@ -543,8 +546,10 @@ int mkv_arena_pair_grow(mkv_arena* k, mkv_arena* v, uint64_t k_add_bytes, uint64
     int rc;
     // the measurement fills two ranges of probe_bytes side by side; under 128 MiB each it no longer tells the
     // groups apart, and a one-sided growth has nothing to separate: plain growth then
+    // Chunks that are no multiple of 2 MiB also grow plainly: candidates are staged back to back, and for a
+    // 574.5 MiB chunk staged at an odd multiple of its size hipMemSetAccess has answered "invalid argument".
     const uint64_t probe_bytes = std::min<uint64_t>(256ull << 20, k->chunk / 2) / 16384 * 16384;
-    if (probe_bytes < (128ull << 20) || need_k == 0 || need_v == 0) {
+    if (probe_bytes < (128ull << 20) || k->chunk % (2ull << 20) != 0 || need_k == 0 || need_v == 0) {
         rc = mkv_arena_resize(k, k->chunks.size() * k->chunk + k_add_bytes);
         if (rc == MKV_OK) {
             rc = mkv_arena_resize(v, v->chunks.size() * v->chunk + v_add_bytes);
