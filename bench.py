@@ -442,7 +442,8 @@ def bench_decode(args):
             round(100.0 * step_bytes / (deferred_graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2) if deferred_graph_ms else None,
         "step_algorithmic_bytes": step_bytes,
         "roofline": {"bound": "hbm",
-                     "kernel": f"attn_decode_phase1_mfma<{HQ // HKV}>" if HQ // HKV >= 4 else f"attn_decode_phase1<{HQ // HKV}>",
+                     "kernel": (f"attn_decode_phase1_mfma<{HQ // HKV}, false>" if HQ // HKV >= 4
+                                else f"attn_decode_phase1<{HQ // HKV}, false>"),
                      "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic(

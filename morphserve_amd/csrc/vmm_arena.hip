@@ -305,22 +305,33 @@ struct PairGrow {
 };
 
 // Split rates measured against one anchor into "same group as the anchor" (slow) and "another group"
-// (fast).  With both kinds present the sorted rates show one wide step (a fifth of the rate on an
-// MI355X); a step under 8 % means one kind only, and the anchor's own rate (its two halves filled side
-// by side: the same group by construction) says which.
+// (fast).  On an MI355X a pair of chunks of one group fills at 4.7-5.8 TB/s and a pair of two groups at
+// 6.0-7.1 TB/s: the two kinds do not overlap, but with a few hundred chunks the gap between them can be as
+// narrow as 6 %, no wider than steps inside a kind are with few chunks.  So the cut is the two-class split
+// of the sorted rates with the largest variance between the classes, and it counts only when the class
+// means lie at least 15 % apart (two kinds: 28 %; one kind cut in two: 10 %); otherwise all rates are of one
+// kind, and the anchor's own rate (its two halves filled side by side: one group by construction) says which.
 static void split_by_rate(const std::vector<double>& rate, double self_rate, std::vector<char>* same) {
     const size_t n = rate.size();
     same->assign(n, 1);
     if (n == 0) return;
     std::vector<double> sorted(rate);
     std::sort(sorted.begin(), sorted.end());
-    double step = 1.0, cut = 0.0;
-    for (size_t i = 0; i + 1 < n; ++i)
-        if (sorted[i + 1] / sorted[i] > step) {
-            step = sorted[i + 1] / sorted[i];
+    double total = 0.0;
+    for (double r : sorted) total += r;
+    double best = -1.0, cut = 0.0, lo_sum = 0.0, ratio = 1.0;
+    for (size_t i = 0; i + 1 < n; ++i) {
+        lo_sum += sorted[i];
+        const double n_lo = (double)(i + 1), n_hi = (double)(n - i - 1);
+        const double m_lo = lo_sum / n_lo, m_hi = (total - lo_sum) / n_hi;
+        const double between = n_lo * n_hi * (m_hi - m_lo) * (m_hi - m_lo);
+        if (between > best) {
+            best = between;
             cut = 0.5 * (sorted[i] + sorted[i + 1]);
+            ratio = m_hi / m_lo;
         }
-    if (step < 1.08) cut = sorted[n / 2] > 1.12 * self_rate ? 0.0 : 1e30;      // all different : all the same
+    }
+    if (ratio < 1.15) cut = sorted[n / 2] > 1.14 * self_rate ? 0.0 : 1e30;      // all different : all the same
     for (size_t i = 0; i < n; ++i) (*same)[i] = rate[i] < cut;
 }
 
