@@ -152,3 +152,44 @@ def test_a_stale_order_is_harmless(cuda):
     want = R.paged_attention(q.cpu().numpy(), case.arena, case.lay, case.block_table, case.seq_ids, shorter.astype(np.int64),
                              128 ** -0.5, 0)
     assert_attn_close(o.cpu().numpy().reshape(n, hq, 128), want, "stale order")
+
+
+def test_order_entries_outside_the_batch_are_clamped(cuda):
+    """The order lives on the device and cannot be checked on the host: the kernels take a slot's own index
+    wherever the entry is not a row of the batch.  All entries out of range -> the rows' own order, bit for
+    bit; some out of range -> every row is either untouched or equal to the plain result."""
+    rng = np.random.default_rng(123)
+    hq, hkv, n, layer = 32, 8, 50, 0
+    lens = rng.integers(1, 400, size=n)
+    case = make_case(11, 1, hq, hkv, lens.tolist(), num_blocks=int(((lens + 15) // 16).sum()) + 2, fill="all")
+    kc, vc, bt = to_gpu(case, cuda)
+    st = build_infer_state([], case.seq_ids.tolist(), lens.tolist(), hkv, 128)
+    q = torch.from_numpy(rand_f16(rng, n, hq, 128)).to(cuda)
+    pool = _capi.make_pool(kc, vc)
+    lib, stream = _capi.lib(), _capi.current_stream()
+    garbage = np.array([n, -1, 10 ** 6, 2 ** 31 - 1, -(2 ** 31), n + 7], dtype=np.int64)
+    all_bad = garbage[rng.integers(0, len(garbage), size=n)].astype(np.int32)
+    some_bad = rng.permutation(n).astype(np.int32)
+    hit = rng.choice(n, size=12, replace=False)
+    some_bad[hit] = garbage[rng.integers(0, len(garbage), size=12)].astype(np.int32)
+    for tps, splits in ((1024, 1), (64, 7)):
+        mid_o = torch.empty(n * hq * splits * 128, dtype=torch.float32, device=cuda)
+        mid_lse = torch.empty(n * hq * splits, dtype=torch.float32, device=cuda)
+        outs = {}
+        for name, order in (("plain", None), ("all_bad", all_bad), ("some_bad", some_bad)):
+            o = torch.full((n, hq * 128), float("nan"), dtype=torch.float16, device=cuda)
+            order_t = torch.from_numpy(order).to(cuda) if order is not None else None
+            _capi.check(lib.mkv_decode_attn_ordered(
+                q.data_ptr(), o.data_ptr(), C.byref(pool), bt.data_ptr(), bt.shape[1], st.seq_ids.data_ptr(),
+                st.decoding_seq_lens.data_ptr(), order_t.data_ptr() if order_t is not None else None, n, hq,
+                128 ** -0.5, layer, tps, splits, mid_o.data_ptr(), mid_lse.data_ptr(), None, None, None, None, stream))
+            torch.cuda.synchronize()
+            outs[name] = bits(o)
+        assert np.array_equal(outs["plain"], outs["all_bad"])
+        for row in hit:         # a slot whose entry is not a row of the batch does its own row
+            assert np.array_equal(outs["some_bad"][row], outs["plain"][row]), row
+        if splits == 1:         # phase 1 writes o itself: a row is either done or was never touched
+            untouched = bits(torch.full((hq * 128,), float("nan"), dtype=torch.float16))
+            for row in range(n):
+                got = outs["some_bad"][row]
+                assert np.array_equal(got, outs["plain"][row]) or np.array_equal(got, untouched), row
