@@ -74,6 +74,12 @@ int mkv_diag_slab_gather(const void* a, const void* b, uint64_t slabs_in_buf, in
 #define MKV_TIMELINE_POINTS 8
 int mkv_diag_timeline(void* buf, int64_t max_workgroups);
 
+/* The rule mkv_arena_pair_grow uses to tell memory groups apart (no counterpart in the reference),
+ * on rates supplied by the caller: rates[i] is the two-stream fill rate of chunk i beside an anchor
+ * chunk, self_rate the anchor's own (its two halves side by side).  same[i] = 1 where chunk i is judged
+ * to lie in the anchor's group.  Host-only: runs without a GPU. */
+int mkv_diag_split_by_rate(const double* rates, int64_t n, double self_rate, uint8_t* same);
+
 /* When enabled, every launch of the kernels above is bracketed by a
  * hipEvent pair on its stream; mkv_prof_collect synchronises those events and
  * returns the launch count and summed duration since the last reset. */

@@ -116,6 +116,7 @@ DIAG_PROTOTYPES = {
     "mkv_diag_mfma_loop": [_I32, _I32, _P, _P, C.POINTER(C.c_double), _P],
     "mkv_diag_timeline": [_P, _I64],
     "mkv_diag_slab_gather": [_P, _P, _U64, _I32, _I32, _I32, _I32, _I32, C.c_uint32, _P, _P],
+    "mkv_diag_split_by_rate": [C.POINTER(C.c_double), _I64, C.c_double, C.POINTER(C.c_uint8)],
     "mkv_prof_enable": [_I32],
     "mkv_prof_reset": [],
     "mkv_prof_collect": [_I32, C.POINTER(_I64), C.POINTER(C.c_double)],

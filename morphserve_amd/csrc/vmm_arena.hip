@@ -591,4 +591,15 @@ int mkv_arena_pair_grow(mkv_arena* k, mkv_arena* v, uint64_t k_add_bytes, uint64
     return rc;
 }
 
+#if MKV_DIAG
+int mkv_diag_split_by_rate(const double* rates, int64_t n, double self_rate, uint8_t* same) {
+    MKV_REQUIRE(rates != nullptr && same != nullptr && n >= 0, "rates and same must not be NULL");
+    std::vector<double> r(rates, rates + n);
+    std::vector<char> out;
+    mkv::split_by_rate(r, self_rate, &out);
+    for (int64_t i = 0; i < n; ++i) same[i] = out[(size_t)i] ? 1 : 0;
+    return MKV_OK;
+}
+#endif
+
 }  // extern "C"

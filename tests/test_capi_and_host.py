@@ -12,7 +12,7 @@ from oracle import ref_cpu as R
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADERS = [os.path.join(ROOT, "include", "morphkv.h"), os.path.join(ROOT, "include", "morphkv_diag.h")]
 DIAG_ONLY = ("mkv_set_decode_variant", "mkv_set_prefill_variant", "mkv_diag_mfma_loop", "mkv_diag_timeline",
-             "mkv_diag_slab_gather", "mkv_prof_enable", "mkv_prof_reset", "mkv_prof_collect")
+             "mkv_diag_slab_gather", "mkv_diag_split_by_rate", "mkv_prof_enable", "mkv_prof_reset", "mkv_prof_collect")
 
 
 def _declared(headers=HEADERS):
