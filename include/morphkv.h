@@ -305,7 +305,10 @@ int mkv_bt_remap(int32_t* block_table, int64_t max_blocks_per_seq,
  * [num_blocks, L, Hkv, B, D] tensor at a fixed address whatever its size, with
  * no extension segments.  mkv_arena_resize maps or unmaps whole chunks at the
  * end (host call; the caller makes sure no kernel still uses memory it gives
- * back); MKV_ENOSPC when the device has no memory left (nothing changed). */
+ * back); MKV_ENOSPC when the device has no memory left (nothing changed).
+ * chunk_bytes: a multiple of the device's allocation granularity, and of 2 MiB when
+ * it is larger than that (chunks are mapped back to back, and the driver has refused
+ * access rights for a 574.5 MiB chunk mapped off a 2 MiB boundary). */
 typedef struct mkv_arena mkv_arena;
 int mkv_arena_create(uint64_t reserve_bytes, uint64_t chunk_bytes, mkv_arena** out);
 int mkv_arena_info(const mkv_arena* arena, void** base, uint64_t* reserved_bytes,
@@ -342,8 +345,7 @@ int mkv_arena_move_tail(mkv_arena* from, mkv_arena* to, uint64_t bytes);
  * while it does).  Where an arena can still grow it also keeps one spare chunk of its group as the
  * reference for later calls (held until mkv_arena_destroy); a later call creates exactly the chunks
  * it needs, measures them against those references and gives each arena the ones of its own group
- * first.  Chunks under 256 MiB cannot be measured, and chunks that are no multiple of 2 MiB cannot be
- * staged for the measurement: plain growth for both.
+ * first.  Chunks under 256 MiB cannot be measured: plain growth.
  * Host call; it synchronises `stream`, on which the measurement kernels run; the new memory holds
  * whatever the measurement left (the caller clears it, as after mkv_arena_resize).  MKV_ENOSPC when
  * the device has no memory left (nothing changed).  `info` (may be NULL) reports what was found. */

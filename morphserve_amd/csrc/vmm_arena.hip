@@ -90,6 +90,11 @@ int mkv_arena_create(uint64_t reserve_bytes, uint64_t chunk_bytes, mkv_arena** o
     *out = nullptr;
     MKV_REQUIRE(chunk_bytes > 0 && reserve_bytes >= chunk_bytes && reserve_bytes % chunk_bytes == 0,
                 "reserve_bytes must be a positive multiple of chunk_bytes");
+    // Chunks are mapped back to back.  A 574.5 MiB chunk mapped at an odd multiple of its size has been
+    // refused by hipMemSetAccess ("invalid argument", the 174th chunk of a range, where the physical
+    // memory crosses from one 96 GiB group of the device into the next); multiples of 2 MiB never were.
+    MKV_REQUIRE(chunk_bytes <= (2ull << 20) || chunk_bytes % (2ull << 20) == 0,
+                "chunk_bytes above 2 MiB must be a multiple of 2 MiB (got %llu)", (unsigned long long)chunk_bytes);
     int dev = 0;
     MKV_HIP(hipGetDevice(&dev));
     int vmm = 0;
@@ -557,10 +562,8 @@ int mkv_arena_pair_grow(mkv_arena* k, mkv_arena* v, uint64_t k_add_bytes, uint64
     int rc;
     // the measurement fills two ranges of probe_bytes side by side; under 128 MiB each it no longer tells the
     // groups apart, and a one-sided growth has nothing to separate: plain growth then
-    // Chunks that are no multiple of 2 MiB also grow plainly: candidates are staged back to back, and for a
-    // 574.5 MiB chunk staged at an odd multiple of its size hipMemSetAccess has answered "invalid argument".
     const uint64_t probe_bytes = std::min<uint64_t>(256ull << 20, k->chunk / 2) / 16384 * 16384;
-    if (probe_bytes < (128ull << 20) || k->chunk % (2ull << 20) != 0 || need_k == 0 || need_v == 0) {
+    if (probe_bytes < (128ull << 20) || need_k == 0 || need_v == 0) {
         rc = mkv_arena_resize(k, k->chunks.size() * k->chunk + k_add_bytes);
         if (rc == MKV_OK) {
             rc = mkv_arena_resize(v, v->chunks.size() * v->chunk + v_add_bytes);

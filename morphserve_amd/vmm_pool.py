@@ -90,7 +90,8 @@ class LayerArena(_Arena):
 
 class VmmKVPool(ElasticKVPool):
     """``num_blocks`` blocks now, room for ``max_blocks``; sizes move in multiples of
-    ``chunk_blocks`` (one physical allocation per chunk and per tensor).
+    ``chunk_blocks`` (one physical allocation per chunk and per tensor; a chunk above 2 MiB must be a
+    multiple of 2 MiB, the library refuses others).
 
     ``placement="groups"`` (the default) lets ``mkv_arena_pair_grow`` choose the physical memory: K chunks
     from one memory group of the device and V chunks from another, told apart by a store-rate measurement

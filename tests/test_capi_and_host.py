@@ -89,6 +89,11 @@ def test_host_only_entry_points():
         _capi.check(lib.mkv_pool_set_strided(ctypes.byref(pool), 0, 0, 1000, 2, 999))
     # argument validation happens before any launch
     assert lib.mkv_append_decode(None, None, None, None, 0, None, None, 1, 0, None) == _capi.MKV_EINVAL
+    # chunk sizes an arena cannot map back to back are refused before the device is touched
+    arena = ctypes.c_void_p()
+    assert lib.mkv_arena_create(12 << 20, 3 << 20, ctypes.byref(arena)) == _capi.MKV_EINVAL
+    assert b"multiple of 2 MiB" in lib.mkv_last_error() and not arena.value
+    assert lib.mkv_arena_create(5 << 20, 2 << 20, ctypes.byref(arena)) == _capi.MKV_EINVAL      # not whole chunks
     with pytest.raises(NotImplementedError):
         swiftllm_c.replace_layer_org2quant(0)
 

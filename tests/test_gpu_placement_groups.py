@@ -23,6 +23,8 @@ GIB = 1 << 30
 
 
 def _free_bytes():
+    import gc
+    gc.collect()                          # pools of earlier tests that are only garbage by now give their memory back here
     torch.cuda.synchronize()
     return torch.cuda.mem_get_info()[0]
 
@@ -43,7 +45,8 @@ def test_group_placed_pool_is_an_ordinary_pool(cuda):
         assert first["candidates"] * CHUNK * (1 << 20) <= 24 * GIB + 2 * CHUNK * (1 << 20)
         # the pool, its two spares and nothing else are held: every other candidate went back
         held = before - _free_bytes()
-        assert 8 * CHUNK * (1 << 20) <= held <= (8 + 2) * CHUNK * (1 << 20) + (512 << 20)
+        slack = 512 << 20                 # torch's own allocator takes and returns memory on the side
+        assert 8 * CHUNK * (1 << 20) - slack <= held <= (8 + 2) * CHUNK * (1 << 20) + slack
         # zero filled whatever the measurement wrote
         assert not pool.k_cache.any() and not pool.v_cache.any()
         # a decode step on it: cache bytes bit-exact, attention within tolerance

@@ -206,6 +206,8 @@ def test_eviction_on_a_virtual_memory_pool(cuda):
 
 # ---- a layer's memory moving into the pool and back ---------------------------------------------------------
 def _free_device_bytes():
+    import gc
+    gc.collect()              # pools of earlier tests that are garbage by now release their memory here, not later
     torch.cuda.synchronize()
     return torch.cuda.mem_get_info()[0]
 

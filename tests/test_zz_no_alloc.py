@@ -48,11 +48,18 @@ def _both_entries(cuda, case, q, layer, tps, splits):
     static_call()             # warm-up: the kernels' code objects are loaded and the scratch address is taken
     # what the DRIVER reports free (hipMemGetInfo), not torch's own counter: an allocation made inside the
     # library (hipMalloc, a memory pool, a virtual-memory mapping) would show here and nowhere else
-    free_before, _ = torch.cuda.mem_get_info()
-    torch_before = torch.cuda.memory_allocated()
-    got.fill_(float("nan"))
-    static_call()
-    free_after, _ = torch.cuda.mem_get_info()
+    import gc
+    gc.collect()              # garbage of earlier tests (pools over virtual memory) gives its memory back now,
+    gc.disable()              # not in the middle of the comparison
+    try:
+        torch.cuda.synchronize()
+        free_before, _ = torch.cuda.mem_get_info()
+        torch_before = torch.cuda.memory_allocated()
+        got.fill_(float("nan"))
+        static_call()
+        free_after, _ = torch.cuda.mem_get_info()
+    finally:
+        gc.enable()
     assert free_after == free_before, f"the call changed the device's free memory by {free_before - free_after} bytes"
     assert torch.cuda.memory_allocated() == torch_before
     return want.cpu().numpy(), got.cpu().numpy()
