@@ -163,20 +163,38 @@ def make_pool(args, num_blocks, max_blocks, L, HKV, B, D, max_seqs, max_blocks_p
 
 
 WIPE_SECONDS_PER_GIB = 0.04
+PROCESS_START = time.perf_counter()
+_wipe_done_at = None          # when the driver will have wiped everything this process knows to have been released
+
+
+def note_release(nbytes):
+    """Memory went back to the driver just now: it is wiped in the background, one release after the other."""
+    global _wipe_done_at
+    now = time.perf_counter()
+    _wipe_done_at = max(_wipe_done_at or now, now) + nbytes / 2 ** 30 * WIPE_SECONDS_PER_GIB
+
+
+def pool_bytes(pool):
+    return 2 * pool.num_blocks * pool.block_bytes
 
 
 def wait_for_driver_wipe(pool):
-    """Pool creation with memory-group placement gives the candidate chunks it did not keep back to the driver,
-    and the driver wipes released memory in the background (about 30 ms per GiB on this system; an allocation
-    that needs such memory waits for it, which is how the rate shows).  While that runs every kernel is a few
-    per cent slower, so a measurement that starts right after pool creation would time the driver's wipe, not
-    the pool.  A server creates its pool long before the first request; the benchmark waits here, for a time
-    computed from the bytes released (nothing is measured or compared to decide it).  Returns the seconds waited."""
-    released = sum(g.get("released_bytes", 0) for g in pool.kv_placement.get("growths", []))
-    wait = released / 2 ** 30 * WIPE_SECONDS_PER_GIB
+    """The driver wipes released memory in the background (about 30 ms per GiB on this system; an allocation
+    that needs such memory waits for it, which is how the rate shows), and while that runs every kernel is a
+    few per cent slower: a measurement that starts right after a release would time the driver's wipe, not the
+    pool.  Releases happen when a pool is created with memory-group placement (the candidate chunks it did
+    not keep), when this program closes a pool, and when a process that ended just before this one gave its
+    memory back, which nothing here can see.  A server creates its pool long before the first request; the
+    benchmark waits here until all of that would be wiped: a time computed from the bytes released and, for
+    the invisible case, from the size of the whole device counted from this process's own start.  Nothing is
+    measured or compared to decide it.  Returns the seconds waited."""
+    import torch
+    note_release(sum(g.get("released_bytes", 0) for g in pool.kv_placement.get("growths", [])))
+    whole_device = PROCESS_START + torch.cuda.mem_get_info()[1] / 2 ** 30 * WIPE_SECONDS_PER_GIB
+    wait = max(_wipe_done_at, whole_device) - time.perf_counter()
     if wait > 0:
         time.sleep(wait)
-    return round(wait, 2)
+    return round(max(wait, 0.0), 2)
 
 
 def diag_kernel_times(fn, kernel_ids):
@@ -462,6 +480,7 @@ def bench_decode(args):
     del graph, k_cache, v_cache
     if hasattr(kv_pool, "close"):
         torch.cuda.synchronize()
+        note_release(pool_bytes(kv_pool))
         kv_pool.close()                           # the memory goes back to the driver before the next workload
     return out
 
@@ -618,9 +637,12 @@ def bench_resize(args, with_cpu_baseline=True):
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    blocks_before = pool.num_blocks
     src, dst = pool.shrink_to(new_n)
     torch.cuda.synchronize()
     shrink_s = time.perf_counter() - t0
+    if hasattr(pool, "close"):                         # a virtual-memory pool gives the tail back to the driver
+        note_release(2 * (blocks_before - new_n) * pool.block_bytes)
     mg_ms = pool.last_migrate_ms
     moves = int(src.numel())
     assert moves == moves_expected
@@ -634,6 +656,7 @@ def bench_resize(args, with_cpu_baseline=True):
     kv_placement = pool.kv_placement
     del src, dst
     if hasattr(pool, "close"):
+        note_release(pool_bytes(pool))
         pool.close()
     cpu = None
     if with_cpu_baseline and not args.no_cpu_baseline:

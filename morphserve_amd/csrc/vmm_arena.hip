@@ -470,7 +470,8 @@ static int pair_grow(PairGrow& g, size_t need_k, size_t need_v, uint64_t budget_
         const size_t want_k = need_k + (k_wants_ref ? 1 : 0), want_v = need_v + (v_wants_ref ? 1 : 0);
         const bool fits = (n0 >= want_k && n1 >= want_v) || (first && n1 >= want_k && n0 >= want_v);
         if (fits || g.cand.size() >= budget_chunks) break;
-        size_t batch = std::min(budget_chunks - g.cand.size(), std::max<size_t>(need / 2, 8));
+        // small steps: every candidate beyond the ones kept goes back to the driver, which wipes it in the background
+        size_t batch = std::min(budget_chunks - g.cand.size(), std::max<size_t>(need / 8, 4));
         if ((rc = g.more(batch, &got))) return rc;
         if (got == 0) break;                                    // the device is full
     }
