@@ -184,6 +184,95 @@ def test_config3_full_size_resize_preserves_logical_kv(cuda):
     assert not is_free[now].any()
 
 
+def test_config3_full_size_resize_on_the_virtual_memory_pool(cuda):
+    """The same resize on the pool the benchmark measures: one tensor per K and V over virtual memory,
+    8 GiB chunks placed by memory group, 32 768 -> 98 304 blocks in eight growths, shrink to 40 960 with the
+    plan made by the multi-workgroup kernels.  Plan, table, free map and counters equal the CPU plan's, every
+    sequence's blocks carry the same bytes afterwards, and the memory above the cut is back with the driver."""
+    if _mem_gib(cuda) < 215:
+        pytest.skip("needs ~200 GiB of free HBM")
+    from morphserve_amd import VmmKVPool
+    L, HKV, D, B = 32, 8, 128, 16
+    ORG, SEG, NSEG, KEEP = 32768, 8192, 8, 1
+    total, new_n = ORG + NSEG * SEG, ORG + KEEP * SEG
+    free_at_start = torch.cuda.mem_get_info(cuda)[0]
+    pool = VmmKVPool(ORG, total, L, HKV, B, D, max_seqs_in_block_table=512, max_blocks_per_seq=256,
+                     chunk_blocks=SEG, placement="groups")
+    try:
+        for _ in range(NSEG):
+            pool.expand(SEG)
+        growths = pool.kv_placement["growths"]
+        assert len(growths) == 1 + NSEG and growths[0]["k_chunks"] == ORG // SEG
+        assert pool.num_blocks == total and pool.k_cache.shape[0] == total
+        assert float(pool.k_cache[ORG + 3 * SEG + 100, 5, 2].abs().sum()) == 0.0          # growth zero-fills
+        rng = np.random.default_rng(33)
+        per_seq, n_seq = 192, 128
+        live = rng.permutation(total)[:per_seq * n_seq]
+        table = np.full((512, 256), -1, dtype=np.int32)
+        n_alloc = np.zeros(512, dtype=np.int32)
+        rows = rng.permutation(512)[:n_seq]
+        for j, s in enumerate(rows):
+            table[s, :per_seq] = live[j * per_seq:(j + 1) * per_seq]
+            n_alloc[s] = per_seq
+        free = np.ones(total, dtype=bool)
+        free[live] = False
+        bm = pool.block_manager
+        bm.block_table.copy_(torch.from_numpy(table))
+        bm.num_seq_allocated_blocks.copy_(torch.from_numpy(n_alloc))
+        bm.is_block_free.copy_(torch.from_numpy(free))
+        bm.num_free_blocks = int(free.sum())
+        bm.invalidate_host_counts()
+
+        gen = torch.Generator(device=cuda)
+        gen.manual_seed(3)
+        weights = torch.arange(1, 4097, dtype=torch.int64, device=cuda)
+        k16 = pool.k_cache.view(torch.int16).reshape(total, -1)
+        v16 = pool.v_cache.view(torch.int16).reshape(total, -1)
+
+        def checksums(ids, kk16, vv16):
+            out = []
+            ids = torch.as_tensor(ids, device=cuda).long()
+            for c0 in range(0, len(ids), 512):
+                sel = ids[c0:c0 + 512]
+                sk = (kk16[sel].view(len(sel), -1, 4096).to(torch.int64) * weights).sum(dim=(1, 2))
+                sv = (vv16[sel].view(len(sel), -1, 4096).to(torch.int64) * weights).sum(dim=(1, 2))
+                out.append(sk * 31 + sv)
+            return torch.cat(out)
+
+        live_t = torch.from_numpy(live).to(cuda).long()
+        for c0 in range(0, len(live), 512):
+            ids = live_t[c0:c0 + 512]
+            pat = torch.randint(-30000, 30000, (len(ids), L * HKV * B * D), dtype=torch.int16, device=cuda, generator=gen)
+            k16[ids] = pat
+            v16[ids] = pat.flip(1)
+        before = checksums(live, k16, v16)
+        want_src, want_dst = R.plan_migration(free, new_n)
+        del k16, v16                                   # views of memory the shrink unmaps
+        src, dst = pool.shrink_to(new_n)
+        torch.cuda.synchronize()
+        assert src.cpu().tolist() == want_src.tolist() and dst.cpu().tolist() == want_dst.tolist()
+        assert pool.num_blocks == new_n and pool.k_cache.shape[0] == new_n
+        new_table = bm.block_table.cpu().numpy()
+        now = np.concatenate([new_table[s, :per_seq] for s in rows])
+        assert now.max() < new_n and len(np.unique(now)) == len(now)
+        remap = dict(zip(want_src.tolist(), want_dst.tolist()))
+        assert np.array_equal(now, np.array([remap.get(int(b), int(b)) for b in live]))
+        k16 = pool.k_cache.view(torch.int16).reshape(new_n, -1)
+        v16 = pool.v_cache.view(torch.int16).reshape(new_n, -1)
+        assert torch.equal(checksums(now, k16, v16), before), "a sequence's KV changed during migration"
+        is_free = bm.is_block_free.cpu().numpy()
+        assert len(is_free) == new_n and int(is_free.sum()) == bm.num_free_blocks == new_n - len(live)
+        assert not is_free[now].any()
+        # the memory above the cut went back to the driver: the pool, its spare chunks and little else are held
+        held = free_at_start - torch.cuda.mem_get_info(cuda)[0]
+        chunk_bytes = SEG * L * HKV * B * D * 2
+        # (torch keeps this test's own temporaries cached: up to a few GiB of gathers and 64-bit sums)
+        assert held <= 2 * (new_n // SEG) * chunk_bytes + 2 * chunk_bytes + (24 << 30) < 2 * (total // SEG) * chunk_bytes
+        del k16, v16
+    finally:
+        pool.close()
+
+
 def test_config5_shapes_one_layer(cuda):
     """CodeLlama-34B decode shapes (GQA 64 q / 8 kv heads, batch 128, contexts in
     [1024, 1536]) on one layer against the CPU oracle."""
