@@ -440,8 +440,9 @@ def bench_decode(args):
                                  else "the grid takes the rows as given (a split batch needs no order)" if _balanced_order()
                                  else "the grid takes the rows as given"),
                    "pool_creation": f"outside the timed region, {pool_creation_s:.2f} s (kv_placement says what the "
-                                    f"memory-group measurement found), then {wiped_s} s for the driver to wipe the "
-                                    "candidate memory that creation gave back"},
+                                    f"memory-group measurement found), then {wiped_s} s of waiting for the driver to "
+                                    "have wiped what was released before (creation's unused candidates, pools this "
+                                    "program closed, at most the whole device by a process that ended just before)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "kv_placement": kv_placement,
         "decode_tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
