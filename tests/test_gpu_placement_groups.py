@@ -113,3 +113,30 @@ def test_plain_placement_and_small_chunks_take_the_drivers_order(cuda):
     with pytest.raises(ValueError):
         VmmKVPool(64, 128, 2, 2, B, D, max_seqs_in_block_table=4, max_blocks_per_seq=8, chunk_blocks=16,
                   placement="nearest")
+
+
+def test_a_pool_that_does_not_fit_is_refused_and_leaves_nothing_behind(cuda):
+    """Device nearly full: creation raises MemoryError (MKV_ENOSPC from the library), every candidate chunk
+    it had created is back with the driver, and the same pool can be created once there is room."""
+    from morphserve_amd.vmm_pool import _Arena
+    free = _free_bytes()
+    if free < 40 * GIB:
+        pytest.skip("needs 40 GiB of free device memory")
+    hog_bytes = (free - 12 * GIB) // GIB * GIB              # leave about 12 GiB
+    hog = _Arena(hog_bytes, GIB)
+    try:
+        hog.resize(hog_bytes)
+        before = _free_bytes()
+        assert before < 14 * GIB
+        with pytest.raises(MemoryError):                    # 2 x 8 GiB in 512 MiB chunks: more than what is left
+            VmmKVPool(16 * CHUNK, 16 * CHUNK, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=64,
+                      chunk_blocks=CHUNK, placement="groups")
+        assert abs(before - _free_bytes()) <= (64 << 20)
+    finally:
+        hog.close()
+    pool = VmmKVPool(16 * CHUNK, 16 * CHUNK, L, HKV, B, D, max_seqs_in_block_table=8, max_blocks_per_seq=64,
+                     chunk_blocks=CHUNK, placement="groups")
+    try:
+        assert pool.kv_placement["growths"][0]["k_chunks"] == 16 and not pool.v_cache[-1].any()
+    finally:
+        pool.close()
